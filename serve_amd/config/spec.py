@@ -48,6 +48,9 @@ class RunEntry:
     layer: int
     cache: int
     writes_cache: bool = True
+    # row of the model's table of pass vectors (`ModelSpec.pass_vectors`) that is added to the residual stream
+    # right before this entry runs (a group of layers that runs several times marks each pass this way)
+    pass_vector: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -65,6 +68,8 @@ class ModelSpec:
     # checkpoint tensors that may be present and are ignored (e.g. stored rotary tables)
     ignored_weight_patterns: List[str] = field(default_factory=list)
     eos_token_ids: Optional[List[int]] = None
+    # a part of role "stream_input" that owns a table [rows, hidden_size]; `RunEntry.pass_vector` names its rows
+    pass_vectors: Optional[PartSpec] = None
 
     def num_cache_layers(self) -> int:
         return 1 + max((e.cache for e in self.run_order), default=-1)

@@ -49,6 +49,8 @@ SOURCES: Dict[str, str] = {
     "latent": "latent.hip",
     "moe": "moe.hip",
     "qk_norm": "qk_norm.hip",
+    "recurrent_scan": "recurrent_scan.hip",
+    "stream_ops": "stream_ops.hip",
 }
 # what a library is linked with beside the HIP runtime
 LINK: Dict[str, List[str]] = {"blaslt.hip": ["-lhipblaslt"]}

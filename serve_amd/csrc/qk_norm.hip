@@ -242,3 +242,148 @@ extern "C" int sa_qk_norm_kv_write(const void* qkv, int row_stride, void* q_out,
   SA_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same place in a mixer whose queries and keys are normed over the whole projection and then rotated:
+//
+//   q[t, :] = N(q[t, :]) * wq   over all Hq D values of the token at once (wq fp32 [Hq D]);  k likewise (wk fp32 [Hk D])
+//   then in every head the first `rot` dims are rotated by the position: dim i pairs with i + rot/2,
+//   (u, v) -> (u cos a - v sin a, v cos a + u sin a), a = position * freq[i]
+//
+// Input rows [Hq D | Hk D | Hk Dv | ...]; outputs as above: q_out [T, Hq Dp], keys and values into the token's slot,
+// every head padded with zeros up to Dp.  Blocks 0 .. T-1 take a token's queries and keys (two sums over the block,
+// then an element a thread at a time); the blocks behind them take the values, a thread per (token, kv head, dim)
+// with tokens fastest, so that writes into the transposed value pages fall into common lines.
+// EXACT: sincosf of the float32 path; else the reduced-argument hardware sine and cosine.
+// ---------------------------------------------------------------------------------------------
+template <typename TA, bool EXACT>
+__global__ __launch_bounds__(256) void row_norm_rope_kv_write_kernel(
+    const TA* __restrict__ qkv, long long row_stride, TA* __restrict__ q_out, const int* __restrict__ positions,
+    const int* __restrict__ slot, TA* __restrict__ k_pages, TA* __restrict__ v_pages, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const float* __restrict__ freq, int rot, int T, int Hq, int Hk, int D,
+    int Dv, int Dp, int page_size) {
+  __shared__ float scratch[16];
+  const TA zero = from_float<TA>(0.f);
+  if ((int)blockIdx.x < T) {
+    const int t = blockIdx.x;
+    const TA* row = qkv + (size_t)t * row_stride;
+    const int nq = Hq * D, nk = Hk * D;
+    float sq = 0.f, sk = 0.f;
+    for (int e = threadIdx.x; e < nq; e += blockDim.x) {
+      const float v = to_float(row[e]);
+      sq = fmaf(v, v, sq);
+    }
+    for (int e = threadIdx.x; e < nk; e += blockDim.x) {
+      const float v = to_float(row[nq + e]);
+      sk = fmaf(v, v, sk);
+    }
+    sq = block_sum(sq, scratch);
+    sk = block_sum(sk, scratch);
+    const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
+    const float pos = (float)positions[t];
+    const int s = slot ? slot[t] : -1;
+    const int page = s >= 0 ? s / page_size : 0, off = s >= 0 ? s - page * page_size : 0;
+    const int half = rot >> 1;
+    const int total = (Hq + (s >= 0 ? Hk : 0)) * Dp;
+    for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+      const int u = idx / Dp, i = idx - u * Dp;
+      const bool is_q = u < Hq;
+      const int g = is_q ? u : u - Hq;
+      TA* dst = is_q ? q_out + ((size_t)t * Hq + g) * Dp : k_pages + (((size_t)page * Hk + g) * page_size + off) * Dp;
+      TA out = zero;
+      if (i < D) {
+        const TA* x = row + (is_q ? 0 : nq) + (size_t)g * D;
+        const float* w = (is_q ? wq : wk) + (size_t)g * D;
+        const float rs = is_q ? rq : rk;
+        float val = (to_float(x[i]) * rs) * w[i];
+        if (i < rot) {
+          const int j = i < half ? i : i - half;
+          const int ip = i < half ? i + half : i - half;
+          const float other = (to_float(x[ip]) * rs) * w[ip];
+          const float a = pos * freq[j];
+          float sn, cs;
+          if (EXACT) sincosf(a, &sn, &cs);
+          else sincos_reduced(a, &sn, &cs);
+          val = i < half ? val * cs - other * sn : val * cs + other * sn;
+        }
+        out = from_float<TA>(val);
+      }
+      dst[i] = out;
+    }
+    return;
+  }
+  if (!slot) return;
+  const long long idx = (long long)(blockIdx.x - T) * 256 + threadIdx.x;
+  if (idx >= (long long)T * Hk * Dp) return;
+  const int t = (int)(idx % T);
+  const int gi = (int)(idx / T);
+  const int g = gi / Dp, i = gi - g * Dp;
+  const int s = slot[t];
+  if (s < 0) return;
+  const int page = s / page_size, off = s - page * page_size;
+  TA out = zero;
+  if (i < Dv) out = qkv[(size_t)t * row_stride + (size_t)(Hq + Hk) * D + (size_t)g * Dv + i];
+  v_pages[(((size_t)page * Hk + g) * Dp + i) * page_size + off] = out;
+}
+
+extern "C" int sa_row_norm_rope_kv_write(const void* qkv, long long row_stride, void* q_out, int act_dtype,
+                                         const int* positions, const int* slot, void* k_pages, void* v_pages,
+                                         const float* wq, const float* wk, float eps, const float* freq, int rot, int T,
+                                         int Hq, int Hk, int D, int Dv, int Dp, int page_size, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (Hq <= 0 || Hk <= 0 || D <= 0 || Dv <= 0 || Dp < D || Dp < Dv || page_size <= 0 || !wq || !wk || !q_out || !positions)
+    return SA_ERR_ARG;
+  if (row_stride < (long long)Hq * D + (long long)Hk * (D + Dv) || (slot && (!k_pages || !v_pages)) || rot < 0 || rot % 2 ||
+      rot > D || (rot > 0 && !freq))
+    return SA_ERR_ARG;
+  const long long v_blocks = slot ? ((long long)T * Hk * Dp + 255) / 256 : 0;
+  if ((long long)T + v_blocks > 0x7fffffffLL) return SA_ERR_ARG;
+  dim3 grid((unsigned)(T + v_blocks)), block(256);
+  if (act_dtype == SA_F32)
+    hipLaunchKernelGGL((row_norm_rope_kv_write_kernel<float, true>), grid, block, 0, stream, (const float*)qkv, row_stride,
+                       (float*)q_out, positions, slot, (float*)k_pages, (float*)v_pages, wq, wk, eps, freq, rot, T, Hq, Hk,
+                       D, Dv, Dp, page_size);
+  else if (act_dtype == SA_BF16)
+    hipLaunchKernelGGL((row_norm_rope_kv_write_kernel<bf16_t, false>), grid, block, 0, stream, (const bf16_t*)qkv,
+                       row_stride, (bf16_t*)q_out, positions, slot, (bf16_t*)k_pages, (bf16_t*)v_pages, wq, wk, eps, freq,
+                       rot, T, Hq, Hk, D, Dv, Dp, page_size);
+  else
+    return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// An output gate per head: a[t, h, :] *= sigmoid(g[t, h]), a [T, H Dp] in place; g: rows of g_stride elements, the
+// heads' logits from column g_col on.
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256) void head_gate_kernel(TA* __restrict__ a, const TA* __restrict__ g, long long g_stride,
+                                                        int g_col, long long total, int H, int Dp) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const long long th = idx / Dp;
+  const long long t = th / H;
+  const int h = (int)(th - t * H);
+  const float z = to_float(g[(size_t)t * g_stride + g_col + h]);
+  a[idx] = from_float<TA>(to_float(a[idx]) * (1.f / (1.f + expf(-z))));
+}
+
+extern "C" int sa_head_gate(void* a, const void* g, int dtype, long long g_stride, int g_col, int T, int H, int Dp,
+                            hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (!a || !g || H <= 0 || Dp <= 0 || g_col < 0) return SA_ERR_ARG;
+  const long long total = (long long)T * H * Dp;
+  const long long blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffLL) return SA_ERR_ARG;
+  if (dtype == SA_F32)
+    hipLaunchKernelGGL(head_gate_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)a, (const float*)g,
+                       g_stride, g_col, total, H, Dp);
+  else if (dtype == SA_BF16)
+    hipLaunchKernelGGL(head_gate_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)a, (const bf16_t*)g,
+                       g_stride, g_col, total, H, Dp);
+  else
+    return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

@@ -38,6 +38,7 @@ class Model:
         self.embedding = _make("embedding", spec.embedding)
         self.final_norm = _make("norm", spec.final_norm)
         self.lm_head = _make("lm_head", spec.lm_head)
+        self.pass_vectors = None if spec.pass_vectors is None else _make("stream_input", spec.pass_vectors)
         self.layers = []
         for i, ls in enumerate(spec.layers):
             arrangement = get_part("arrangement", ls.arrangement)
@@ -50,6 +51,8 @@ class Model:
         for e in spec.run_order:
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"run order names layer {e.layer}, the model has {len(self.layers)}")
+            if e.pass_vector is not None and self.pass_vectors is None:
+                raise ValueError("the run order names a pass vector, the model has no table of them")
         self._check_cache_owners()
         self.rt: Optional[Runtime] = None
 
@@ -57,6 +60,8 @@ class Model:
     def _owners(self) -> Dict[str, Part]:
         owners: Dict[str, Part] = {"embedding": self.embedding, "final_norm": self.final_norm,
                                    "lm_head": self.lm_head}
+        if self.pass_vectors is not None:
+            owners["pass_vectors"] = self.pass_vectors
         for i, layer in enumerate(self.layers):
             for name, part in layer.parts().items():
                 owners[f"layers.{i}.{name}"] = part
@@ -74,6 +79,8 @@ class Model:
                                          pr.alias_of, pr.alias_only))
 
         add("embedding", self.embedding, self.spec.weights, "embedding.")
+        if self.pass_vectors is not None:
+            add("pass_vectors", self.pass_vectors, self.spec.weights, "pass_vectors.")
         for i, (layer, ls) in enumerate(zip(self.layers, self.spec.layers)):
             for name, part in layer.parts().items():
                 add(f"layers.{i}.{name}", part, ls.weights, name + ".")
@@ -174,6 +181,10 @@ class Model:
             # end of its own last kernel and leave the result in ctx.shared
             nxt = self.layers[order[i + 1].layer] if i + 1 < len(order) else None
             ctx.next_input_norm = nxt.input_norm() if hasattr(nxt, "input_norm") else None
+            if nxt is not None and order[i + 1].pass_vector is not None:
+                ctx.next_input_norm = None          # (the stream changes between the two layers)
+            if e.pass_vector is not None:
+                pending = self.pass_vectors.forward(x, pending, e.pass_vector)
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)

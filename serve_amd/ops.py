@@ -611,6 +611,289 @@ def qk_norm_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Te
     return q_out
 
 
+def row_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                           slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                           v_pages: Optional[torch.Tensor], q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float,
+                           inv_freq: Optional[torch.Tensor], rot_dim: int, num_heads: int, num_kv_heads: int, dim: int,
+                           vdim: int) -> torch.Tensor:
+    """From rows qkv [T, Hq D | Hk D | Hk Dv | ...]: all queries of a token over their common root mean square (eps
+    inside the root) times `q_weight` (fp32 [Hq D]), all its keys likewise with `k_weight` (fp32 [Hk D]); then in every
+    head the first `rot_dim` dims rotated by position * inv_freq[i] (dim i paired with i + rot_dim / 2).  Queries go
+    to q_out [T, Hq Dp], keys and values to the token's slot of k_pages [P, Hk, page, Dp] and v_pages
+    [P, Hk, Dp, page], each head padded with zeros up to Dp.  `slots` None: queries only."""
+    _dev(q_out, positions, slots, k_pages, v_pages, q_weight, k_weight, inv_freq)
+    Hq, Hk, D, Dv = num_heads, num_kv_heads, dim, vdim
+    T = qkv.shape[0]
+    _check(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= Hq * D + Hk * (D + Dv),
+           f"qkv must be rows of at least {Hq * D + Hk * (D + Dv)} on the GPU")
+    _check(q_out.dim() == 2 and q_out.shape[0] == T and q_out.shape[1] % Hq == 0 and q_out.dtype == qkv.dtype,
+           "q_out must be [T, Hq Dp] in the dtype of qkv")
+    Dp = q_out.shape[1] // Hq
+    _check(Dp >= D and Dp >= Dv, f"the padded head size {Dp} is below dim {D} or vdim {Dv}")
+    _f32vec(q_weight, Hq * D, "q norm weight")
+    _f32vec(k_weight, Hk * D, "k norm weight")
+    _check(rot_dim >= 0 and rot_dim % 2 == 0 and rot_dim <= D, "rot_dim must be even and within dim")
+    if rot_dim:
+        _f32vec(inv_freq, rot_dim // 2, "inv_freq")
+    _i32(positions, T, "positions")
+    page_size = 1
+    if slots is not None:
+        _i32(slots, T, "slots")
+        P, _, page_size, _ = k_pages.shape
+        _check(k_pages.shape == (P, Hk, page_size, Dp) and v_pages.shape == (P, Hk, Dp, page_size),
+               f"the cache must be k [P, {Hk}, page, {Dp}] and v [P, {Hk}, {Dp}, page]")
+        _check(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "cache dtype must match activations")
+    lib = load_library("qk_norm")
+    _ret(lib.sa_row_norm_rope_kv_write(_ptr(qkv), ctypes.c_longlong(qkv.stride(0)), _ptr(q_out), c_int(_code(qkv)),
+                                       _ptr(positions), _ptr(slots), _ptr(k_pages if slots is not None else None),
+                                       _ptr(v_pages if slots is not None else None), _ptr(q_weight), _ptr(k_weight),
+                                       c_float(eps), _ptr(inv_freq if rot_dim else None), c_int(rot_dim), c_int(T),
+                                       c_int(Hq), c_int(Hk), c_int(D), c_int(Dv), c_int(Dp), c_int(page_size),
+                                       _stream()), "row_norm_rope_kv_write")
+    return q_out
+
+
+def head_gate(a: torch.Tensor, rows: torch.Tensor, col: int, num_heads: int) -> torch.Tensor:
+    """a[t, h, :] *= sigmoid(rows[t, col + h]) in place: a [T, H Dp], the heads' gate logits in the columns
+    col .. col + H - 1 of `rows` (which may be a wider product's output)."""
+    _dev(a)
+    T = a.shape[0]
+    _check(a.dim() == 2 and a.shape[1] % num_heads == 0, "a must be [T, H Dp]")
+    _check(rows.is_cuda and rows.device == a.device and rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[0] == T
+           and rows.dtype == a.dtype and 0 <= col and col + num_heads <= rows.shape[1],
+           "the gate logits must be columns of [T, >= col + H] rows in a's dtype")
+    lib = load_library("qk_norm")
+    _ret(lib.sa_head_gate(_ptr(a), _ptr(rows), c_int(_code(a)), ctypes.c_longlong(rows.stride(0)), c_int(col), c_int(T),
+                          c_int(num_heads), c_int(a.shape[1] // num_heads), _stream()), "head_gate")
+    return a
+
+
+# ---------------------------------------------------------------------------------------------
+# around the residual stream
+# ---------------------------------------------------------------------------------------------
+
+def _parts_of(y: torch.Tensor, T: int, d: int, what: str):
+    if y.dim() == 3:
+        _check(y.dtype == torch.float32 and y.shape[1:] == (T, d), f"{what}: partial sums must be fp32 [parts, T, d]")
+        return y.shape[0]
+    _check(y.shape == (T, d), f"{what} must be [T, d]")
+    return 1
+
+
+def stream_add(x: torch.Tensor, y: Optional[torch.Tensor], vec: Optional[torch.Tensor] = None,
+               h: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += y + vec on the fp32 residual stream x [T, d], in place (y: [T, d] or fp32 [parts, T, d] partial sums, added
+    in order; vec fp32 [d]; either may be None), and `h` ([T, d], any kernel dtype) receives a copy of the new x."""
+    _dev(x, y, vec, h)
+    _check(x.dtype == torch.float32 and x.dim() == 2, "residual stream must be fp32 [T, d]")
+    T, d = x.shape
+    parts, ycode = 1, F32
+    if y is not None:
+        parts, ycode = _parts_of(y, T, d, "y"), _code(y)
+    if vec is not None:
+        _f32vec(vec, d, "the row vector")
+    if h is not None:
+        _check(h.shape == (T, d), "the stream's copy must be [T, d]")
+    lib = load_library("stream_ops")
+    _ret(lib.sa_stream_add(_ptr(x), _ptr(y), c_int(ycode), c_int(parts), _ptr(vec), _ptr(h),
+                           c_int(_code(h) if h is not None else F32), c_int(T), c_int(d), _stream()), "stream_add")
+    return h
+
+
+def dual_norm_mix(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, ca: float, cb: float,
+                  eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out = ca N(a) wa + cb N(b) wb per row, N(y) = y / sqrt(mean(y^2) + eps); a and b [T, d] or fp32 [parts, T, d]
+    partial sums; wa, wb fp32 [d]; out fp32 [T, d]."""
+    _dev(a, b, wa, wb, out)
+    _check(out.dtype == torch.float32 and out.dim() == 2, "the mixed output must be fp32 [T, d]")
+    T, d = out.shape
+    pa, pb = _parts_of(a, T, d, "a"), _parts_of(b, T, d, "b")
+    _f32vec(wa, d, "the first norm's weight")
+    _f32vec(wb, d, "the second norm's weight")
+    lib = load_library("stream_ops")
+    _ret(lib.sa_dual_norm_mix(_ptr(a), c_int(_code(a)), c_int(pa), _ptr(b), c_int(_code(b)), c_int(pb), _ptr(wa), _ptr(wb),
+                              c_float(ca), c_float(cb), c_float(eps), _ptr(out), c_int(T), c_int(d), _stream()),
+         "dual_norm_mix")
+    return out
+
+
+def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, col: int, tokens: torch.Tensor, out: torch.Tensor,
+                  src_row: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, j] = gelu_tanh(z[t, j]) * table[token_t, col + j] for z [T, n]; the token of row t is tokens[t], or
+    prev[src_row[t]] where src_row[t] >= 0 (a token sampled on the device by an earlier step)."""
+    _dev(z, table, tokens, out, src_row, prev)
+    _check(z.dim() == 2 and out.shape == z.shape and out.dtype == z.dtype, "z and out must be [T, n] of one dtype")
+    T, n = z.shape
+    _check(table.dim() == 2 and 0 <= col and col + n <= table.shape[1], "the table must be [V, >= col + n]")
+    _i32(tokens, T, "tokens")
+    if src_row is not None:
+        _i32(src_row, T, "src_row")
+        _check(prev is not None and prev.dtype == torch.int32, "prev must be int32")
+    lib = load_library("stream_ops")
+    _ret(lib.sa_gelu_mul_rows(_ptr(z), c_int(_code(z)), _ptr(table), c_int(_code(table)),
+                              ctypes.c_longlong(table.shape[1]), c_int(col), _ptr(tokens), _ptr(src_row), _ptr(prev),
+                              _ptr(out), c_int(T), c_int(n), c_int(table.shape[0]), _stream()), "gelu_mul_rows")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# recurrences S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t
+# ---------------------------------------------------------------------------------------------
+SCAN_MAX_DIM = 256
+SCAN_MAX_TAPS = 16
+
+
+def decay_scan_state_floats(heads: int, dk: int, dv: int) -> int:
+    """Floats of a request's state row that `decay_scan` keeps for `heads` matrices [dk, dv]: the kernel's own
+    layout, rows padded to 16 x a power of two and columns to whole tiles (csrc/recurrent_scan.hip)."""
+    if not (heads > 0 and 0 < dk <= SCAN_MAX_DIM and dv > 0):
+        raise KernelError(f"decay_scan takes key sizes up to {SCAN_MAX_DIM}; got heads {heads}, dk {dk}, dv {dv}")
+    rpt = 1
+    while 16 * rpt < dk:
+        rpt *= 2
+    cpt = 4 if dv >= 64 else (2 if dv >= 32 else 1)
+    tiles = -(-dv // (16 * cpt))
+    return heads * tiles * rpt * 256 * cpt
+
+
+def _rows(t: torch.Tensor, T: int, width: int, name: str) -> None:
+    _check(t.is_cuda and t.dim() == 2 and t.shape[0] == T and t.stride(1) == 1 and t.shape[1] >= width,
+           f"{name} must be rows [T, >= {width}] on the GPU")
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+               state_offset: int, ctx, out: torch.Tensor, heads: int, qk_heads: int, dk: int, dv: int,
+               q_scale: float = 1.0) -> torch.Tensor:
+    """Per segment of the step and head h, from the request's state S (fp32, zeros for a new request), token by token:
+    S = diag(a) S + k v^T, out = S^T (q_scale q).  q, k: rows [T, >= qk_heads dk] (views with a row stride are fine;
+    head h reads q/k head h // (heads / qk_heads)); v rows [T, >= heads dv]; all three of one dtype.  decay fp32
+    [T, heads, dk] (one per key channel) or [T, heads] (one per head).  state fp32 [slots, row]: the matrices live at
+    `state_offset` of a request's row (ctx.state_slots, -1: none) in the kernel's own layout
+    (`decay_scan_state_floats` floats).  out fp32 [T, heads dv]."""
+    T, B = ctx.num_tokens, ctx.num_segments
+    _dev(decay, out, ctx.cu_q, ctx.state_slots)
+    _check(heads % qk_heads == 0 and 0 < dk <= SCAN_MAX_DIM and dv > 0, "decay_scan: heads must be a multiple of qk_heads, dk <= 256")
+    _rows(q, T, qk_heads * dk, "q")
+    _rows(k, T, qk_heads * dk, "k")
+    _rows(v, T, heads * dv, "v")
+    _check(q.dtype == k.dtype == v.dtype and q.device == k.device == v.device == out.device, "q, k and v must share dtype and device")
+    per_channel = decay.dim() == 3
+    _check(decay.dtype == torch.float32 and tuple(decay.shape) in ((T, heads, dk), (T, heads)),
+           "decay must be fp32 [T, H, dk] or [T, H]")
+    _check(out.dtype == torch.float32 and out.shape == (T, heads * dv), "out must be fp32 [T, H dv]")
+    need = decay_scan_state_floats(heads, dk, dv)
+    _check(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+           and 0 <= state_offset and state_offset + need <= state.shape[1],
+           f"state rows must be fp32 with {need} floats from offset {state_offset}")
+    _i32(ctx.cu_q, B + 1, "cu_q")
+    _i32(ctx.state_slots, B, "state_slots")
+    lib = load_library("recurrent_scan")
+    LL = ctypes.c_longlong
+    _ret(lib.sa_decay_scan(_ptr(q), _ptr(k), _ptr(v), c_int(_code(q)), LL(q.stride(0)), LL(k.stride(0)), LL(v.stride(0)),
+                           _ptr(decay), c_int(1 if per_channel else 0), c_float(q_scale),
+                           c_void_p(state.data_ptr() + 4 * state_offset), LL(state.stride(0)), _ptr(ctx.cu_q),
+                           _ptr(ctx.state_slots), _ptr(out), c_int(B), c_int(heads), c_int(qk_heads), c_int(dk), c_int(dv),
+                           _stream()), "decay_scan")
+    return out
+
+
+def gla_decay(z: torch.Tensor, bias: Optional[torch.Tensor], tau: float, out: torch.Tensor) -> torch.Tensor:
+    """out = sigmoid(z + bias)^(1 / tau), computed as exp(ln sigmoid(.) / tau): z, out fp32 [T, C], bias fp32 [C]."""
+    _dev(z, bias, out)
+    _check(z.dtype == torch.float32 and z.dim() == 2 and out.shape == z.shape and out.dtype == torch.float32,
+           "decay logits and decays must be fp32 [T, C]")
+    if bias is not None:
+        _f32vec(bias, z.shape[1], "the decay's bias")
+    _check(tau > 0, "tau must be positive")
+    lib = load_library("recurrent_scan")
+    _ret(lib.sa_gla_decay(_ptr(z), _ptr(bias), c_float(tau), _ptr(out), c_int(z.shape[0]), c_int(z.shape[1]), _stream()),
+         "gla_decay")
+    return out
+
+
+def ssm_prepare(zx: torch.Tensor, col: int, conv_w: torch.Tensor, conv_b: Optional[torch.Tensor], state: torch.Tensor,
+                conv_offset: int, dt_raw: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, ctx,
+                xbc: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, heads: int, head_dim: int, taps: int) -> None:
+    """The state-space mixer's inputs.  zx rows [T, >= col + C]: columns col .. col + C - 1 are the convolution's
+    channels [x: H P | B | C]; conv_w fp32 [C, taps] (last column on the current token), conv_b fp32 [C] or None;
+    inputs before a segment come from its request's state row at `conv_offset` ([taps - 1, C] fp32, oldest first).
+    xbc fp32 [T, C] = silu(conv); dt = softplus(dt_raw + dt_bias) (dt_raw fp32 [T, H]); decay fp32 [T, H] =
+    exp(-exp(A_log) dt); v fp32 [T, H P] = dt x."""
+    T, B = ctx.num_tokens, ctx.num_segments
+    _dev(conv_w, conv_b, dt_raw, A_log, dt_bias, xbc, v, decay, ctx.seg_of_token, ctx.cu_q, ctx.state_slots)
+    H, P = heads, head_dim
+    _check(xbc.dtype == torch.float32 and xbc.dim() == 2 and xbc.shape[0] == T, "xbc must be fp32 [T, C]")
+    C = xbc.shape[1]
+    _check(C >= H * P and 1 <= taps <= SCAN_MAX_TAPS, f"channels must cover H P = {H * P}; up to {SCAN_MAX_TAPS} taps")
+    _rows(zx, T, col + C, "zx")
+    _check(conv_w.dtype == torch.float32 and conv_w.shape == (C, taps), f"conv_w must be fp32 [{C}, {taps}]")
+    if conv_b is not None:
+        _f32vec(conv_b, C, "conv bias")
+    _check(dt_raw.dtype == torch.float32 and dt_raw.shape == (T, H), "dt_raw must be fp32 [T, H]")
+    _f32vec(A_log, H, "A_log")
+    _f32vec(dt_bias, H, "dt_bias")
+    _check(v.dtype == torch.float32 and v.shape == (T, H * P) and decay.dtype == torch.float32 and decay.shape == (T, H),
+           "v must be fp32 [T, H P] and decay fp32 [T, H]")
+    _check(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+           and 0 <= conv_offset and conv_offset + (taps - 1) * C <= state.shape[1], "state rows are too short for the convolution")
+    _i32(ctx.seg_of_token, T, "seg_of_token")
+    _i32(ctx.cu_q, B + 1, "cu_q")
+    _i32(ctx.state_slots, B, "state_slots")
+    lib = load_library("recurrent_scan")
+    LL = ctypes.c_longlong
+    _ret(lib.sa_ssm_prepare(_ptr(zx), c_int(_code(zx)), LL(zx.stride(0)), c_int(col), _ptr(conv_w), _ptr(conv_b),
+                            _ptr(state), LL(state.stride(0)), LL(conv_offset), _ptr(dt_raw), _ptr(A_log), _ptr(dt_bias),
+                            _ptr(ctx.seg_of_token), _ptr(ctx.cu_q), _ptr(ctx.state_slots), _ptr(xbc), _ptr(v), _ptr(decay),
+                            c_int(T), c_int(H), c_int(P), c_int(C), c_int(taps), _stream()), "ssm_prepare")
+
+
+def conv_state_update(zx: torch.Tensor, col: int, channels: int, state: torch.Tensor, conv_offset: int, ctx,
+                      taps: int) -> None:
+    """After a step: the last taps - 1 inputs of every channel (columns col .. col + channels - 1 of zx rows) into the
+    requests' state rows at `conv_offset`, oldest first; a segment shorter than taps - 1 keeps the newest of its old ones."""
+    T, B = ctx.num_tokens, ctx.num_segments
+    _dev(ctx.cu_q, ctx.state_slots)
+    _rows(zx, T, col + channels, "zx")
+    _check(1 <= taps <= SCAN_MAX_TAPS, f"up to {SCAN_MAX_TAPS} taps")
+    _check(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+           and 0 <= conv_offset and conv_offset + (taps - 1) * channels <= state.shape[1], "state rows are too short for the convolution")
+    _i32(ctx.cu_q, B + 1, "cu_q")
+    _i32(ctx.state_slots, B, "state_slots")
+    lib = load_library("recurrent_scan")
+    LL = ctypes.c_longlong
+    _ret(lib.sa_conv_state_update(_ptr(zx), c_int(_code(zx)), LL(zx.stride(0)), c_int(col), _ptr(state), LL(state.stride(0)),
+                                  LL(conv_offset), _ptr(ctx.cu_q), _ptr(ctx.state_slots), c_int(B), c_int(channels),
+                                  c_int(taps), _stream()), "conv_state_update")
+
+
+def gated_group_norm(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, weight: torch.Tensor, group: int,
+                     gate_first: bool, eps: float, out: torch.Tensor, skip_x: Optional[torch.Tensor] = None,
+                     skip_d: Optional[torch.Tensor] = None, head_dim: int = 1) -> torch.Tensor:
+    """What follows a recurrence's read-out o fp32 [T, n]: u = o + skip_d[i // head_dim] skip_x[t, i] (skip_x fp32 rows
+    [T, >= n], or None); with g = silu(gate_rows[t, gate_col + i]): `gate_first`: out = N(u g) w, else out = N(u) w g,
+    where N divides every run of `group` values by its root mean square (eps inside the root) and w = weight[i % len]."""
+    _dev(o, weight, out, skip_d)
+    _check(o.dtype == torch.float32 and o.dim() == 2, "o must be fp32 [T, n]")
+    T, n = o.shape
+    _check(group > 0 and n % group == 0, f"groups of {group} do not divide {n}")
+    _check(out.shape == (T, n) and out.dtype == gate_rows.dtype, "out must be [T, n] in the gate's dtype")
+    _rows(gate_rows, T, gate_col + n, "gate rows")
+    _check(weight.dtype == torch.float32 and weight.dim() == 1 and weight.numel() > 0, "the norm's weight must be an fp32 vector")
+    skip_stride = 0
+    if skip_x is not None:
+        _rows(skip_x, T, n, "skip_x")
+        _check(skip_x.dtype == torch.float32 and skip_d is not None and head_dim > 0 and n % head_dim == 0, "skip_x must be fp32 rows with skip_d")
+        _f32vec(skip_d, n // head_dim, "skip_d")
+        skip_stride = skip_x.stride(0)
+    lib = load_library("recurrent_scan")
+    LL = ctypes.c_longlong
+    _ret(lib.sa_gated_group_norm(_ptr(o), _ptr(skip_x), LL(skip_stride), _ptr(skip_d), c_int(head_dim), _ptr(gate_rows),
+                                 c_int(_code(gate_rows)), LL(gate_rows.stride(0)), c_int(gate_col), _ptr(weight),
+                                 c_int(weight.numel()), c_int(group), c_int(1 if gate_first else 0), c_float(eps), _ptr(out),
+                                 c_int(T), c_int(n), _stream()), "gated_group_norm")
+    return out
+
+
 # ---------------------------------------------------------------------------------------------
 # routed experts
 # ---------------------------------------------------------------------------------------------

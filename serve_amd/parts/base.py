@@ -44,7 +44,7 @@ class ParamRequest:
     embedding table."""
 
     name: str
-    shape: Tuple[int, ...]
+    shape: Tuple[int, ...]          # (-1: a size that only the checkpoint's tensor gives; the loader takes any)
     # how the random-weights writer fills it: "normal" = N(0, 0.02), "ones_normal" = 1 + N(0, 0.1)
     init: str = "normal"
     optional: bool = False
@@ -178,7 +178,7 @@ class Part:
         for pr in self.param_requests():
             n = 1
             for d in pr.shape:
-                n *= int(d)
+                n *= max(int(d), 0)         # (a size that only the checkpoint gives counts as nothing)
             elements += n               # (a tensor that is another part's, an alias, is still read here)
             if len(pr.shape) == 2:
                 flops += 2.0 * tokens * n

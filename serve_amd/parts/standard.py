@@ -271,17 +271,24 @@ class TokenEmbedding(Part):
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, side_width: int = 0):
         """`scale` multiplies every row as it enters the stream (in fp32; the table itself, which an
-        output head may share, stays as stored)."""
+        output head may share, stays as stored).  `side_width` > 0: the part also holds a second table
+        `side` [vocab, side_width], a second row per token that parts of the layers read (they name it as
+        `embedding.side`); nothing of it enters the stream here."""
         self.vocab_size, self.hidden_size, self.scale = int(vocab_size), int(hidden_size), float(scale)
+        self.side_width = int(side_width)
 
     def param_requests(self) -> List[ParamRequest]:
-        return [ParamRequest("weight", (self.vocab_size, self.hidden_size))]
+        out = [ParamRequest("weight", (self.vocab_size, self.hidden_size))]
+        if self.side_width:
+            out.append(ParamRequest("side", (self.vocab_size, self.side_width), init="normal:1.0"))
+        return out
 
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         self.weight = tensors["weight"]
+        self.side = tensors.get("side")
 
     def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
         """A gather of `tokens` rows: no product, and of the table only those rows are read (not
@@ -336,25 +343,43 @@ class PreNormResidual:
     """x = x + mixer(norm1(x)); x = x + ffn(norm2(x)) (serve/model.py:146-149).
 
     The additions are folded into the following norm: `pending` is the output of the previous
-    part that has not been added to the residual stream yet; the layer returns its own."""
+    part that has not been added to the residual stream yet; the layer returns its own.
 
-    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "ffn_norm": "norm"}
+    A layer may have no feed-forward (then it has no `ffn_norm` either), and it may end with a
+    `token_input`: a part that adds something made from the step's tokens and the finished stream
+    (`forward(x, pending, ctx) -> pending`: it folds the layer's last output into x itself)."""
 
-    def __init__(self, mixer, ffn, mixer_norm, ffn_norm):
+    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "ffn_norm": "norm",
+                  "token_input": "token_input"}
+    OPTIONAL_PARTS = ("ffn", "ffn_norm", "token_input")
+
+    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None, token_input=None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+        self.token_input = token_input
 
     def cache_owner(self) -> Part:
         return self.mixer
 
     def parts(self) -> Dict[str, Part]:
-        return {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}
+        out = {"mixer": self.mixer, "mixer_norm": self.mixer_norm}
+        if self.ffn is not None:
+            out.update(ffn=self.ffn, ffn_norm=self.ffn_norm)
+        if self.token_input is not None:
+            out["token_input"] = self.token_input
+        return out
 
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
-                writes_cache: bool = True) -> torch.Tensor:
+                writes_cache: bool = True) -> Optional[torch.Tensor]:
         h = self.mixer_norm.forward(x, pending)
         a = self.mixer.forward(h, ctx, cache, writes_cache)
-        h = self.ffn_norm.forward(x, a)
-        return self.ffn.forward(h, ctx)
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(x, a)
+            a = self.ffn.forward(h, ctx)
+        if self.token_input is not None:
+            a = self.token_input.forward(x, a, ctx)
+        return a
 
 
 register_part("norm", "rmsnorm", RMSNorm)

@@ -1,0 +1,89 @@
+"""Inputs to the residual stream beside the token embedding.
+
+`GatedSideEmbedding` (role `token_input`, the last part of a layer): with e the layer's slice of a second embedding
+row of the token, and x the stream after the layer's sublayers,
+
+    g = gelu_tanh(W_gate x) * e;    y = W_proj g;    x <- x + y / sqrt(mean(y^2) + eps) * w
+
+The second table is the embedding part's (`embedding.side`); a layer reads the columns [offset, offset + dim).
+
+`PassVectors` (role `stream_input`, a part of the model): a table [rows, width] of which the run order adds one row to
+the stream before an entry runs.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from ..registry import register_part
+from .base import ParamRequest, Part, Runtime, StepCost
+from .linear import linear
+
+
+class GatedSideEmbedding(Part):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, vocab_size: int, table_width: int, offset: int, dim: int, eps: float):
+        if not 0 <= offset and offset + dim <= table_width:
+            raise ValueError(f"columns [{offset}, {offset + dim}) do not lie in a table of width {table_width}")
+        self.hidden_size, self.vocab_size, self.table_width = int(hidden_size), int(vocab_size), int(table_width)
+        self.offset, self.dim, self.eps = int(offset), int(dim), float(eps)
+
+    def param_requests(self) -> List[ParamRequest]:
+        d, n = self.hidden_size, self.dim
+        return [ParamRequest("gate", (n, d), init="normal:0.08"), ParamRequest("proj", (d, n), init="normal:0.08"),
+                ParamRequest("norm", (d,), init="ones_normal"),
+                ParamRequest("table", (self.vocab_size, self.table_width), alias_of="embedding.side", alias_only=True)]
+
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        """The two small products; of the table only the tokens' rows are read."""
+        n = 2 * self.dim * self.hidden_size
+        return StepCost(n + self.hidden_size, 2.0 * tokens * n)
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.w_gate, self.w_proj, self.table = tensors["gate"], tensors["proj"], tensors["table"]
+        self.norm_w = tensors["norm"].float().contiguous()
+        self.ones = torch.ones((self.hidden_size,), dtype=torch.float32, device=rt.device)
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx) -> Optional[torch.Tensor]:
+        """Fold `pending` (the layer's last output) into the stream, then add this part's own.  Returns what is
+        still to be added: nothing."""
+        xc = self.rt.empty(tuple(x.shape))
+        ops.stream_add(x, pending, None, xc)
+        z = linear(xc, self.w_gate)
+        g = ops.gelu_mul_rows(z, self.table, self.offset, ctx.token_ids, self.rt.empty(tuple(z.shape)), ctx.src_row,
+                              ctx.prev_tokens)
+        y = linear(g, self.w_proj, partial_ok=True)
+        ops.output_norm_add(x, y, self.norm_w, self.ones, self.eps, None)
+        return None
+
+
+class PassVectors(Part):
+    graph_safe = True
+
+    def __init__(self, rows: int, hidden_size: int):
+        self.rows, self.hidden_size = int(rows), int(hidden_size)
+
+    def param_requests(self) -> List[ParamRequest]:
+        return [ParamRequest("weight", (self.rows, self.hidden_size), init="normal:0.3")]
+
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        return StepCost(0, 0.0)
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.table = tensors["weight"].float().contiguous()          # the stream is fp32
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], row: int) -> Optional[torch.Tensor]:
+        """x += pending + table[row]; nothing is left to be added."""
+        if not 0 <= row < self.rows:
+            raise ValueError(f"pass vector {row} of {self.rows}")
+        ops.stream_add(x, pending, self.table[row], None)
+        return None
+
+
+register_part("token_input", "gated_side_embedding", GatedSideEmbedding)
+register_part("stream_input", "pass_vectors", PassVectors)

@@ -24,7 +24,8 @@ class Architecture:
 _ARCHITECTURES: Dict[str, Architecture] = {}
 _PARTS: Dict[Tuple[str, str], type] = {}
 
-PART_ROLES = ("mixer", "feed_forward", "norm", "position", "embedding", "lm_head", "arrangement")
+PART_ROLES = ("mixer", "feed_forward", "norm", "position", "embedding", "lm_head", "arrangement", "token_input",
+              "stream_input")
 
 
 def register_architecture(name: str, config_from_dict, build_spec) -> None:
@@ -84,3 +85,4 @@ def _ensure_builtin() -> None:
         from .models import llama  # noqa: F401  (registers LlamaForCausalLM)
         from .models import zozosun  # noqa: F401  (registers Zozosun)
         from .models import timopel  # noqa: F401  (registers Timopel)
+        from .models import kotipel  # noqa: F401  (registers Kotipel)

@@ -61,7 +61,7 @@ def check_against(model: Model, reader) -> List[WeightRequest]:
                 missing.append(r.checkpoint_name)
             continue
         _, shape = reader.info(r.checkpoint_name)
-        if tuple(shape) != tuple(r.shape):
+        if len(shape) != len(r.shape) or any(w not in (-1, int(g)) for g, w in zip(shape, r.shape)):
             wrong.append((r.checkpoint_name, tuple(shape), tuple(r.shape)))
         else:
             present.append(r)
@@ -110,6 +110,9 @@ def random_tensors(model: Model, seed: int, dtype: torch.dtype = torch.bfloat16,
     for r in model.weight_requests():
         if r.alias_only:
             continue
+        if any(n < 0 for n in r.shape):
+            raise ValueError(f"the shape of {r.checkpoint_name} {list(r.shape)} is the checkpoint's to say: a model with "
+                             "random weights needs the size in its configuration")
         g = torch.Generator(device="cpu")
         g.manual_seed(_tensor_seed(seed, r.checkpoint_name))
         t = torch.randn(r.shape, generator=g, dtype=torch.float32)
