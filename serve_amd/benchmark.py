@@ -102,8 +102,34 @@ SHAPES.update({
     "timopel-2k": _timopel_shape(2048, 32768, 8, 32, 8, 64, 8192, 32, 4, 1024, 2048),
     "timopel-4k": _timopel_shape(4096, 32768, 4, 32, 8, 128, 14336, 64, 6, 1536, 3072),
 })
+
+
+def _kotipel_shape(width: int, vocab: int, layers: int, loop, heads: int, kv_heads: int, head: int, lin_heads: int,
+                   lin_dim: int, lin_vdim: int, ssm_heads: int, ssm_groups: int, ff: int, side: int):
+    """A Kotipel shape at the sizes of a real model's layers: in turn a parallel layer (softmax attention with `heads` on
+    `kv_heads` heads of `head`, half of whose dims are rotated, beside a gated linear attention of `lin_heads` heads of
+    `lin_dim` x `lin_vdim`) and a state-space layer (inner width twice the model's: `ssm_heads` heads of 64, state 128,
+    four taps), each with a clamped feed-forward of `ff` and a token input of `side`; `loop` = (start, stop, times)."""
+    from .config.kotipel import (ClampedDenseConfig, GatedAttentionConfig, KotipelConfig, KotipelLayerConfig,
+                                 LinearAttentionConfig, LoopConfig, ParallelMixerConfig, RotScaling, StateSpaceMixerConfig)
+    par = ParallelMixerConfig(
+        GatedAttentionConfig(heads, kv_heads, head, head, head ** -0.5, head // 2, 500000.0, RotScaling(8.0, 1.0, 4.0, 8192.0)),
+        LinearAttentionConfig(lin_heads, lin_dim, lin_vdim, 16.0, 16))
+    ssm = StateSpaceMixerConfig(ssm_heads, 64, 128, ssm_groups, 4, 1)
+    mlp = ClampedDenseConfig(ff, 7.0)
+    return KotipelConfig(vocab=vocab, width=width, eps=1e-5, loop=LoopConfig(*loop), side_dim=side,
+                         layers=tuple(KotipelLayerConfig(par if i % 2 == 0 else ssm, mlp) for i in range(layers)))
+
+
+# Kotipel at the same two widths, vocabularies, attention head shapes and feed-forward widths; with the layers that
+# run twice it has as many layer runs as the Llama shapes have layers (8 and 4)
+SHAPES.update({
+    "kotipel-tiny": _kotipel_shape(64, 512, 2, (0, 2, 2), 4, 2, 16, 2, 16, 32, 2, 1, 128, 8),
+    "kotipel-2k": _kotipel_shape(2048, 32768, 6, (2, 4, 2), 32, 8, 64, 16, 64, 128, 64, 1, 8192, 256),
+    "kotipel-4k": _kotipel_shape(4096, 32768, 3, (1, 2, 2), 32, 8, 128, 16, 128, 256, 128, 8, 14336, 256),
+})
 DESIGN_PAIRS = (("zozosun-2k", "llama-2k"), ("zozosun-4k", "llama-4k"), ("timopel-2k", "llama-2k"),
-                ("timopel-4k", "llama-4k"))
+                ("timopel-4k", "llama-4k"), ("kotipel-2k", "llama-2k"), ("kotipel-4k", "llama-4k"))
 
 
 def generate_requests(input_length: int, output_length: int, num_sequences: int, vocab_size: int,
