@@ -5,9 +5,12 @@
 // A gated linear attention is this with a decay per key channel; a selective state-space mixer with S [state, head dim],
 // k = B_t, q = C_t, v = dt_t x_t and the one decay exp(-exp(A_log) dt_t) a head.  What differs between such mixers lies
 // in front of the recurrence (how q, k, v and the decays are made) and behind it (norm and gate of the read-out), so the
-// file has the recurrence itself (`decay_scan`), the two preparations (`gla_decay`; `ssm_prepare` with the causal
-// convolution, and `conv_state_update` for the convolution's last inputs) and one kernel for what follows (`gated_group_norm`).
-// All arithmetic is fp32; template types are the storage of projections and outputs.
+// file has the recurrence itself (`decay_scan`: token by token for single tokens and short portions, sixteen tokens a
+// pass on the matrix cores for prompts), the two preparations (`gla_decay`; `ssm_prepare` with the causal convolution,
+// and `conv_state_update` for the convolution's last inputs) and one kernel for what follows (`gated_group_norm`).
+// The decays travel as their logarithms (<= 0), which is how both preparations get them and what a pass over several
+// tokens sums.  All arithmetic is fp32, also on the matrix cores (v_mfma_f32_16x16x4_f32); template types are the
+// storage of projections and outputs.
 #include "common.h"
 
 #define RS_MAX_TAPS 16
@@ -44,7 +47,7 @@ __device__ __forceinline__ float row16_sum(float v) {
 template <typename TQ, int RPT, int CPT, int CH>
 __global__ __launch_bounds__(256) void decay_scan_kernel(
     const TQ* __restrict__ q, const TQ* __restrict__ k, const TQ* __restrict__ v, long long q_stride,
-    long long k_stride, long long v_stride, const float* __restrict__ decay, int per_channel, float q_scale,
+    long long k_stride, long long v_stride, const float* __restrict__ log_decay, int per_channel, float q_scale,
     float* __restrict__ state, long long state_stride, const int* __restrict__ cu_q,
     const int* __restrict__ state_slots, float* __restrict__ o, int H, int Hk, int dk, int dv) {
   constexpr int ROWS = 16 * RPT;
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
       const int ic = in ? i : 0;
       const float qv = to_float(q[tok * q_stride + (size_t)hk * dk + ic]) * q_scale;
       const float kv = to_float(k[tok * k_stride + (size_t)hk * dk + ic]);
-      const float av = per_channel ? decay[(tok * H + h) * (size_t)dk + ic] : decay[tok * H + h];
+      const float av = expf(per_channel ? log_decay[(tok * H + h) * (size_t)dk + ic] : log_decay[tok * H + h]);
       sq[tt][pos] = in ? qv : 0.f;
       sk[tt][pos] = in ? kv : 0.f;
       sa[tt][pos] = in ? av : 1.f;
@@ -180,20 +183,233 @@ static void launch_scan_r(int rpt, int cpt, const void* q, const void* k, const 
 #undef GO
 }
 
+// ---------------------------------------------------------------------------------------------
+// The recurrence for prompts: sixteen tokens a pass.  With b_t the sum of the logarithms of the decays of tokens
+// 0..t of the pass (a vector over the key channels, <= 0 and falling) and S0 the state before it:
+//
+//   o_t = S0^T (q_t e^(b_t))  +  sum_(s<=t) A[t, s] v_s          A[t, s] = sum_c q_t[c] k_s[c] e^(b_t[c] - b_s[c])
+//   S   = diag(e^(b_15)) S0   +  sum_s (k_s e^(b_15 - b_s)) v_s^T
+//
+// Both lines are matrix products of fp32 operands (v_mfma_f32_16x16x4_f32, fp32 in and out), and every factor
+// e^(..) in them is at most 1.  A too is a product, (q_t e^(b_t - b_7)) . (k_s e^(b_7 - b_s)), as long as no channel
+// decays by more than e^-80 within either half of the pass, so that neither factor leaves the range of fp32; a pass
+// where one does sums the channels of each of its 136 entries one by one, with the exponent of the difference
+// itself.  A pass that the segment's end cuts short is filled with tokens that change nothing (q = k = v = 0,
+// decay 1).
+//
+// grid (ceil(dv / 64), H, B), 256 threads: wave w owns 16 columns and keeps their S in the registers of the matrix
+// cores' result layout (lane (g, j): rows 16 m + 4 g + r, column j), which serves as the second operand of
+// S0^T q directly when the contraction runs over the rows in that same order.  All waves share the scaled q and k
+// of the pass in LDS; the next pass's inputs are loaded into registers while this one's products run.  A request's
+// state is read and written in the token-by-token kernel's layout (RPT, CPT: its row and column split), since a
+// request changes between the two with every step.
+// ---------------------------------------------------------------------------------------------
+typedef float rs_f4 __attribute__((ext_vector_type(4)));
+#define RS_RANGE 80.f
+
+template <typename TQ, int NT>
+__global__ __launch_bounds__(256) void decay_scan_block_kernel(
+    const TQ* __restrict__ q, const TQ* __restrict__ k, const TQ* __restrict__ v, long long q_stride,
+    long long k_stride, long long v_stride, const float* __restrict__ log_decay, int per_channel, float q_scale,
+    float* __restrict__ state, long long state_stride, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slots, float* __restrict__ o, int H, int Hk, int dk, int dv, int RPT, int CPT) {
+  constexpr int DKP = 16 * NT;                   // the key channels, padded
+  constexpr int ST = DKP + 4;                    // row stride in LDS: 4 (or 20) mod 32 banks, and rows stay 16-byte aligned
+  constexpr int NE = NT;                         // q / k elements of a pass per thread: 16 DKP / 256
+  __shared__ __attribute__((aligned(16))) float sb[16][ST];     // b_t
+  __shared__ __attribute__((aligned(16))) float sqh[16][ST];    // q e^(b_t)
+  __shared__ __attribute__((aligned(16))) float skt[16][ST];    // k e^(b_15 - b_t)
+  __shared__ __attribute__((aligned(16))) float sqp[16][ST];    // q e^(b_t - b_7), or q itself
+  __shared__ __attribute__((aligned(16))) float skp[16][ST];    // k e^(b_7 - b_t), or k itself
+  __shared__ __attribute__((aligned(16))) float sdec[DKP];      // e^(b_15)
+  __shared__ float sv[16][68];
+  __shared__ float sap[4][16][17];
+  __shared__ float sam[16][20];
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, j = lane & 15;
+  const int tile = blockIdx.x, h = blockIdx.y, seg = blockIdx.z;
+  const int hk = h / (H / Hk);
+  const int slot = state_slots[seg];
+  const int t0 = cu_q[seg], n = cu_q[seg + 1] - t0;
+  if (n <= 0) return;
+  const int col = tile * 64 + w * 16 + j;        // this lane's column of S and o
+  const int seq_tiles = (dv + 16 * CPT - 1) / (16 * CPT);
+  // where the token-by-token kernel keeps (row, col) of head h
+  auto state_at = [&](int row) -> size_t {
+    return (((size_t)h * seq_tiles + col / (16 * CPT)) * RPT + row % RPT) * (size_t)(256 * CPT) +
+           (size_t)(((col / CPT) % 16) * 16 + row / RPT) * CPT + col % CPT;
+  };
+  float* st = slot >= 0 && col < dv ? state + (size_t)slot * state_stride : nullptr;
+  rs_f4 S[NT];
+#pragma unroll
+  for (int m = 0; m < NT; ++m)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) S[m][r] = st ? st[state_at(16 * m + 4 * g + r)] : 0.f;
+
+  // the inputs of a pass, in registers: log decays (threads below DKP: one channel each), q, k, v
+  float rla[16], rq[NE], rk[NE], rv[4];
+  auto fetch = [&](int c0) {
+    const int m = min(16, n - c0);
+    if (tid < DKP) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const size_t tok = (size_t)(t0 + c0 + t);
+        rla[t] = (t < m && tid < dk) ? (per_channel ? log_decay[(tok * H + h) * (size_t)dk + tid] : log_decay[tok * H + h]) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      const int idx = tid + 256 * e, t = idx / DKP, c = idx % DKP;
+      const bool in = t < m && c < dk;
+      const size_t tok = (size_t)(t0 + c0 + t);
+      rq[e] = in ? to_float(q[tok * q_stride + (size_t)hk * dk + c]) * q_scale : 0.f;
+      rk[e] = in ? to_float(k[tok * k_stride + (size_t)hk * dk + c]) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int idx = tid + 256 * e, t = idx >> 6, c = idx & 63;
+      const int jj = tile * 64 + c;
+      rv[e] = (t < m && jj < dv) ? to_float(v[(size_t)(t0 + c0 + t) * v_stride + (size_t)h * dv + jj]) : 0.f;
+    }
+  };
+  fetch(0);
+  for (int c0 = 0; c0 < n; c0 += 16) {
+    const int m = min(16, n - c0);
+    __syncthreads();                             // the pass before has read its LDS
+    int far = 0;
+    if (tid < DKP) {
+      float run = 0.f, b7 = 0.f;
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        run += rla[t];
+        sb[t][tid] = run;
+        if (t == 7) b7 = run;
+      }
+      sdec[tid] = expf(run);
+      far = (b7 < -RS_RANGE) || (run - b7 < -RS_RANGE);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int idx = tid + 256 * e;
+      sv[idx >> 6][idx & 63] = rv[e];
+    }
+    const int wide = __syncthreads_or(far);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+      const int idx = tid + 256 * e, t = idx / DKP, c = idx % DKP;
+      const float bt = sb[t][c], b7 = sb[7][c], b15 = sb[15][c];
+      sqh[t][c] = rq[e] * expf(bt);
+      skt[t][c] = rk[e] * expf(b15 - bt);
+      sqp[t][c] = wide ? rq[e] : rq[e] * expf(bt - b7);
+      skp[t][c] = wide ? rk[e] : rk[e] * expf(b7 - bt);
+    }
+    if (c0 + 16 < n) fetch(c0 + 16);             // in flight while the products run
+    __syncthreads();
+    // A, the weights of the pass's own tokens
+    if (!wide) {
+      rs_f4 acc = {0.f, 0.f, 0.f, 0.f};
+      const int cb = w * 4 * NT;                 // each wave a quarter of the channels
+#pragma unroll
+      for (int s4 = 0; s4 < NT; ++s4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(sqp[j][cb + 4 * s4 + g], skp[j][cb + 4 * s4 + g], acc, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sap[w][4 * g + r][j] = acc[r];
+      __syncthreads();
+      const int t = tid >> 4, s = tid & 15;
+      sam[t][s] = s <= t ? (sap[0][t][s] + sap[1][t][s]) + (sap[2][t][s] + sap[3][t][s]) : 0.f;
+    } else {
+      const int t = tid >> 4, s = tid & 15;
+      float a = 0.f;
+      if (s <= t)
+        for (int c = 0; c < DKP; ++c) a = fmaf(sqp[t][c] * skp[s][c], expf(sb[t][c] - sb[s][c]), a);
+      sam[t][s] = a;
+    }
+    __syncthreads();
+    // this wave's 16 columns: the read-out ...
+    float vb[4];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) vb[s4] = sv[4 * s4 + g][w * 16 + j];
+    rs_f4 oc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < NT; ++mt) {
+      const rs_f4 a4 = *reinterpret_cast<const rs_f4*>(&sqh[j][16 * mt + 4 * g]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], S[mt][r], oc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(sam[j][4 * s4 + g], vb[s4], oc, 0, 0, 0);
+    if (col < dv) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (4 * g + r < m) o[((size_t)(t0 + c0 + 4 * g + r) * H + h) * dv + col] = oc[r];
+    }
+    // ... and the state after the pass
+#pragma unroll
+    for (int mt = 0; mt < NT; ++mt) {
+      const rs_f4 d4 = *reinterpret_cast<const rs_f4*>(&sdec[16 * mt + 4 * g]);
+      rs_f4 sm = S[mt];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sm[r] *= d4[r];
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) sm = __builtin_amdgcn_mfma_f32_16x16x4f32(skt[4 * s4 + g][16 * mt + j], vb[s4], sm, 0, 0, 0);
+      S[mt] = sm;
+    }
+  }
+  if (st) {
+#pragma unroll
+    for (int m = 0; m < NT; ++m)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) st[state_at(16 * m + 4 * g + r)] = S[m][r];
+  }
+}
+
+template <typename TQ>
+static int launch_scan_block(int rpt, int cpt, const void* q, const void* k, const void* v, long long qs, long long ks,
+                             long long vs, const float* decay, int per_channel, float q_scale, float* state,
+                             long long state_stride, const int* cu_q, const int* slots, float* o, int B, int H, int Hk,
+                             int dk, int dv, hipStream_t stream) {
+  dim3 grid((dv + 63) / 64, H, B), block(256);
+#define GO(N) hipLaunchKernelGGL((decay_scan_block_kernel<TQ, N>), grid, block, 0, stream, (const TQ*)q, (const TQ*)k, (const TQ*)v, qs, ks, vs, decay, per_channel, q_scale, state, state_stride, cu_q, slots, o, H, Hk, dk, dv, rpt, cpt)
+  switch (rpt) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 4: GO(4); break;
+    case 8: GO(8); break;
+    default: return SA_ERR_UNSUPPORTED;
+  }
+#undef GO
+  return 0;
+}
+
+// the longest segment from which a launch takes sixteen tokens a pass, and the widest key it does so for
+#define RS_BLOCK_MIN_TOKENS 6
+#define RS_BLOCK_MAX_DK 128
+extern "C" int sa_decay_scan_block_min_tokens() { return RS_BLOCK_MIN_TOKENS; }
+
 // q, k: rows of `q_stride` / `k_stride` elements with head hk's dk values at hk dk (Hk heads; head h reads hk = h / (H / Hk));
-// v: rows of `v_stride` with head h's dv values at h dv; decay fp32 [T, H, dk] (per_channel) or [T, H]; o fp32 [T, H, dv];
+// v: rows of `v_stride` with head h's dv values at h dv; decay: the decays' logarithms, fp32 [T, H, dk] (per_channel) or [T, H];
+// o fp32 [T, H, dv]; max_q: the longest segment (what decides between the two kernels);
 // state: a request's row at state + slot state_stride (the floats that sa_decay_scan_state_floats counts), slot < 0: a
 // segment without a request, which starts from zeros and keeps nothing.
 extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dtype, long long q_stride,
                              long long k_stride, long long v_stride, const float* decay, int per_channel,
                              float q_scale, float* state, long long state_stride, const int* cu_q,
-                             const int* state_slots, float* o, int B, int H, int Hk, int dk, int dv,
+                             const int* state_slots, float* o, int B, int H, int Hk, int dk, int dv, int max_q,
                              hipStream_t stream) {
   if (B <= 0) return 0;
   if (H <= 0 || Hk <= 0 || H % Hk || dk <= 0 || dk > 256 || dv <= 0 || !q || !k || !v || !decay || !state || !o ||
       !cu_q || !state_slots || B > 65535 || H > 65535)
     return SA_ERR_ARG;
   const int rpt = scan_rpt(dk), cpt = scan_cpt(dv);
+  if (max_q >= RS_BLOCK_MIN_TOKENS && dk <= RS_BLOCK_MAX_DK && (dtype == SA_F32 || dtype == SA_BF16)) {
+    const int rc = dtype == SA_F32
+        ? launch_scan_block<float>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
+                                   state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream)
+        : launch_scan_block<bf16_t>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
+                                    state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream);
+    if (rc) return rc;
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == SA_F32)
     launch_scan_r<float>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
                          state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream);
@@ -207,7 +423,7 @@ extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dt
 }
 
 // ---------------------------------------------------------------------------------------------
-// decay[t, c] = sigmoid(z[t, c] + b[c])^(1 / tau) = exp(ln sigmoid(z + b) / tau), c over H dk channels
+// The logarithm of the decay sigmoid(z[t, c] + b[c])^(1 / tau):  ln sigmoid(z + b) / tau, c over H dk channels
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict__ z, const float* __restrict__ bias,
                                                         float inv_tau, float* __restrict__ decay, long long total,
@@ -215,7 +431,7 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict_
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
   const int c = (int)(idx % C);
-  decay[idx] = expf(rs_logsigmoid(z[idx] + (bias ? bias[c] : 0.f)) * inv_tau);
+  decay[idx] = rs_logsigmoid(z[idx] + (bias ? bias[c] : 0.f)) * inv_tau;
 }
 
 extern "C" int sa_gla_decay(const float* z, const float* bias, float tau, float* decay, int T, int C,
@@ -235,7 +451,7 @@ extern "C" int sa_gla_decay(const float* z, const float* bias, float tau, float*
 // convolution's channels [x: H P | B: G N | C: G N].  Per token and channel: the causal convolution over `taps` inputs
 // (w [C, taps], the last column on the current token, bias b; inputs before the segment come from the request's state
 // row at conv_off, [taps - 1, C] oldest first, or are zeros where the segment has no request) and silu -> xbc fp32 [T, C].
-// Per token and head: dt = softplus(dtraw + dt_bias), decay = exp(-exp(A_log) dt); v = dt x -> fp32 [T, H P].
+// Per token and head: dt = softplus(dtraw + dt_bias), the decay's logarithm -exp(A_log) dt -> decay [T, H]; v = dt x -> fp32 [T, H P].
 // grid (T, ceil((C + H) / 256)).
 // ---------------------------------------------------------------------------------------------
 template <typename TA>
@@ -251,7 +467,7 @@ __global__ __launch_bounds__(256) void ssm_prepare_kernel(
   if (c >= C) {
     const int h = c - C;
     const float dt = rs_softplus(dtraw[(size_t)t * H + h] + dt_bias[h]);
-    decay[(size_t)t * H + h] = expf(-expf(A_log[h]) * dt);
+    decay[(size_t)t * H + h] = -expf(A_log[h]) * dt;
     return;
   }
   const int seg = seg_of_token[t];
@@ -353,22 +569,26 @@ extern "C" int sa_conv_state_update(const void* zx, int dtype, long long zs, int
 //   else:        y = u / sqrt(mean_group(u^2) + eps) * w[i % wn] * silu(g[t, i])
 // g: rows of gate_stride elements in the output's storage type, read from column gate_col on.
 // ---------------------------------------------------------------------------------------------
-template <typename TA>
+// WAVES: how many waves share a group (1: a wave a group, four groups a block; 4: a block a group, for groups of
+// thousands, where a single wave's chain of loads would decide the time of a decode step)
+template <typename TA, int WAVES>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     const float* __restrict__ o, const float* __restrict__ skip_x, long long skip_stride,
     const float* __restrict__ skip_d, int dv, const TA* __restrict__ gate, long long gate_stride, int gate_col,
     const float* __restrict__ w, int wn, int group, int gate_first, float eps, TA* __restrict__ y, long long units,
     int n) {
-  const int lane = threadIdx.x & (SA_WAVE - 1);
-  const long long unit = (long long)blockIdx.x * (256 / SA_WAVE) + threadIdx.x / SA_WAVE;
-  if (unit >= units) return;
+  __shared__ float part[4];
+  constexpr int LANES = SA_WAVE * WAVES;
+  const int lane = threadIdx.x & (LANES - 1);
+  const long long unit = (long long)blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
+  if (unit >= units) return;                    // (whole blocks when WAVES is 4)
   const int groups = n / group;
   const long long t = unit / groups;
   const int i0 = (int)(unit - t * groups) * group;
   const float* orow = o + (size_t)t * n;
   const TA* grow = gate + (size_t)t * gate_stride + gate_col;
   float ss = 0.f;
-  for (int e = lane; e < group; e += SA_WAVE) {
+  for (int e = lane; e < group; e += LANES) {
     const int i = i0 + e;
     float u = orow[i];
     if (skip_x) u = fmaf(skip_d[i / dv], skip_x[(size_t)t * skip_stride + i], u);
@@ -376,8 +596,13 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     ss = fmaf(u, u, ss);
   }
   ss = wave_sum(ss);
+  if (WAVES > 1) {
+    if ((threadIdx.x & (SA_WAVE - 1)) == 0) part[threadIdx.x / SA_WAVE] = ss;
+    __syncthreads();
+    ss = (part[0] + part[1]) + (part[2] + part[3]);
+  }
   const float rs = 1.0f / sqrtf(ss / (float)group + eps);
-  for (int e = lane; e < group; e += SA_WAVE) {
+  for (int e = lane; e < group; e += LANES) {
     const int i = i0 + e;
     float u = orow[i];
     if (skip_x) u = fmaf(skip_d[i / dv], skip_x[(size_t)t * skip_stride + i], u);
@@ -397,17 +622,19 @@ extern "C" int sa_gated_group_norm(const float* o, const float* skip_x, long lon
   if (!o || !gate || !w || !y || n <= 0 || group <= 0 || n % group || wn <= 0 || dv <= 0 || (skip_x && !skip_d))
     return SA_ERR_ARG;
   const long long units = (long long)T * (n / group);
-  const long long blocks = (units + 3) / 4;
+  const bool whole = group >= 512;              // a block a group
+  const long long blocks = whole ? units : (units + 3) / 4;
   if (blocks > 0x7fffffffLL) return SA_ERR_ARG;
   dim3 grid((unsigned)blocks), block(256);
-  if (dtype == SA_F32)
-    hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, o, skip_x, skip_stride, skip_d, dv,
-                       (const float*)gate, gate_stride, gate_col, w, wn, group, gate_first, eps, (float*)y, units, n);
-  else if (dtype == SA_BF16)
-    hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, grid, block, 0, stream, o, skip_x, skip_stride, skip_d, dv,
-                       (const bf16_t*)gate, gate_stride, gate_col, w, wn, group, gate_first, eps, (bf16_t*)y, units, n);
-  else
+#define GO(TA, W) hipLaunchKernelGGL((gated_group_norm_kernel<TA, W>), grid, block, 0, stream, o, skip_x, skip_stride, skip_d, dv, (const TA*)gate, gate_stride, gate_col, w, wn, group, gate_first, eps, (TA*)y, units, n)
+  if (dtype == SA_F32) {
+    if (whole) GO(float, 4); else GO(float, 1);
+  } else if (dtype == SA_BF16) {
+    if (whole) GO(bf16_t, 4); else GO(bf16_t, 1);
+  } else {
     return SA_ERR_UNSUPPORTED;
+  }
+#undef GO
   SA_LAUNCH_CHECK();
   return 0;
 }

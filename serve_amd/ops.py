@@ -741,6 +741,7 @@ def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, col: int, tokens: torch.
 # ---------------------------------------------------------------------------------------------
 SCAN_MAX_DIM = 256
 SCAN_MAX_TAPS = 16
+SCAN_BLOCK_MIN_TOKENS = 6        # csrc/recurrent_scan.hip: RS_BLOCK_MIN_TOKENS
 
 
 def decay_scan_state_floats(heads: int, dk: int, dv: int) -> int:
@@ -766,8 +767,10 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
                q_scale: float = 1.0) -> torch.Tensor:
     """Per segment of the step and head h, from the request's state S (fp32, zeros for a new request), token by token:
     S = diag(a) S + k v^T, out = S^T (q_scale q).  q, k: rows [T, >= qk_heads dk] (views with a row stride are fine;
-    head h reads q/k head h // (heads / qk_heads)); v rows [T, >= heads dv]; all three of one dtype.  decay fp32
-    [T, heads, dk] (one per key channel) or [T, heads] (one per head).  state fp32 [slots, row]: the matrices live at
+    head h reads q/k head h // (heads / qk_heads)); v rows [T, >= heads dv]; all three of one dtype.  decay: ln a, fp32
+    [T, heads, dk] (one per key channel) or [T, heads] (one per head).  A step whose longest segment has
+    `SCAN_BLOCK_MIN_TOKENS` tokens or more takes sixteen tokens a pass on the matrix cores (keys up to 128 wide),
+    any other goes token by token.  state fp32 [slots, row]: the matrices live at
     `state_offset` of a request's row (ctx.state_slots, -1: none) in the kernel's own layout
     (`decay_scan_state_floats` floats).  out fp32 [T, heads dv]."""
     T, B = ctx.num_tokens, ctx.num_segments
@@ -793,12 +796,13 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
                            _ptr(decay), c_int(1 if per_channel else 0), c_float(q_scale),
                            c_void_p(state.data_ptr() + 4 * state_offset), LL(state.stride(0)), _ptr(ctx.cu_q),
                            _ptr(ctx.state_slots), _ptr(out), c_int(B), c_int(heads), c_int(qk_heads), c_int(dk), c_int(dv),
-                           _stream()), "decay_scan")
+                           c_int(int(getattr(ctx, "max_q_len", 0) or T)), _stream()), "decay_scan")
     return out
 
 
 def gla_decay(z: torch.Tensor, bias: Optional[torch.Tensor], tau: float, out: torch.Tensor) -> torch.Tensor:
-    """out = sigmoid(z + bias)^(1 / tau), computed as exp(ln sigmoid(.) / tau): z, out fp32 [T, C], bias fp32 [C]."""
+    """out = ln(sigmoid(z + bias)^(1 / tau)) = ln sigmoid(z + bias) / tau, the decay's logarithm that `decay_scan` takes:
+    z, out fp32 [T, C], bias fp32 [C]."""
     _dev(z, bias, out)
     _check(z.dtype == torch.float32 and z.dim() == 2 and out.shape == z.shape and out.dtype == torch.float32,
            "decay logits and decays must be fp32 [T, C]")
@@ -818,7 +822,7 @@ def ssm_prepare(zx: torch.Tensor, col: int, conv_w: torch.Tensor, conv_b: Option
     channels [x: H P | B | C]; conv_w fp32 [C, taps] (last column on the current token), conv_b fp32 [C] or None;
     inputs before a segment come from its request's state row at `conv_offset` ([taps - 1, C] fp32, oldest first).
     xbc fp32 [T, C] = silu(conv); dt = softplus(dt_raw + dt_bias) (dt_raw fp32 [T, H]); decay fp32 [T, H] =
-    exp(-exp(A_log) dt); v fp32 [T, H P] = dt x."""
+    -exp(A_log) dt, the decay's logarithm; v fp32 [T, H P] = dt x."""
     T, B = ctx.num_tokens, ctx.num_segments
     _dev(conv_w, conv_b, dt_raw, A_log, dt_bias, xbc, v, decay, ctx.seg_of_token, ctx.cu_q, ctx.state_slots)
     H, P = heads, head_dim

@@ -279,24 +279,33 @@ def _ctx(lens, slots):
                            state_slots=torch.tensor(slots, **dev))
 
 
+# steps of two requests and a segment of nobody's: short ones go token by token, the others sixteen tokens a pass
+SCAN_STEPS = {"short": [[4, 1, 3], [1, 5, 2]], "mid": [[9, 1, 3], [1, 21, 2]], "long": [[33, 1, 16], [1, 64, 7], [47, 3, 1]]}
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("per_channel", [True, False])
+@pytest.mark.parametrize("decays", ["mild", "strong"])
+@pytest.mark.parametrize("steps", sorted(SCAN_STEPS))
 @pytest.mark.parametrize("dk,dv,H,Hk", [(16, 32, 4, 2), (32, 64, 2, 2), (10, 70, 1, 1), (48, 20, 3, 1), (130, 16, 2, 1),
-                                        (256, 128, 1, 1), (5, 9, 2, 2)])
-def test_decay_scan_in_two_steps(dk, dv, H, Hk, per_channel, dtype):
-    """Two requests over two steps (one of each as a single token) and a segment without a request, against the plain
-    recurrence over the whole sequences: the state carries over, lies where it is asked to, and nothing else is written."""
+                                        (256, 128, 1, 1), (5, 9, 2, 2), (128, 64, 2, 1), (64, 128, 2, 2)])
+def test_decay_scan_over_steps(dk, dv, H, Hk, per_channel, dtype, steps, decays):
+    """Two requests over several steps (portions, single tokens) and a segment without a request, against the plain
+    recurrence over the whole sequences: the state carries over between the two kernels, lies where it is asked to,
+    and nothing else is written.  `strong`: decays down to e^-30 a token, which a pass of sixteen cannot factor."""
     from serve_amd import ops
     torch.manual_seed(dk + dv)
-    lens = [[9, 1, 3], [1, 21, 2]]                   # request 0: 9 then 1; request 1: 1 then 21; the third belongs to nobody
-    total = [10, 22]
+    lens = SCAN_STEPS[steps]
+    total = [sum(n[0] for n in lens), sum(n[1] for n in lens)]
     rnd = lambda *s: torch.randn(*s).to(dtype).double()   # noqa: E731  (values the storage type holds)
     q = [rnd(n, Hk * dk) for n in total]
     k = [rnd(n, Hk * dk) for n in total]
     v = [rnd(n, H * dv) for n in total]
-    a = [torch.rand(n, H, dk, dtype=torch.float64) * 0.5 + 0.5 if per_channel else torch.rand(n, H, dtype=torch.float64) * 0.5 + 0.5
-         for n in total]
-    a = [x.float().double() for x in a]
+    span = 0.7 if decays == "mild" else 30.0
+    la = [-(torch.rand(n, H, dk, dtype=torch.float64) if per_channel else torch.rand(n, H, dtype=torch.float64)) ** 3 * span
+          for n in total]
+    la = [x.float().double() for x in la]            # the logarithms are what the kernel gets
+    a = [torch.exp(x) for x in la]
     scale = 0.37
     want = []
     for r in range(2):
@@ -307,12 +316,12 @@ def test_decay_scan_in_two_steps(dk, dv, H, Hk, per_channel, dtype):
     off = 7
     state = torch.zeros(3, off + need + 5, dtype=torch.float32, device="cuda")
     at, got = [0, 0], [[], []]
-    for step in range(2):
+    for step in range(len(lens)):
         n = lens[step]
         cat = lambda xs, w: torch.cat([xs[0][at[0]: at[0] + n[0]], xs[1][at[1]: at[1] + n[1]],   # noqa: E731
                                        torch.ones(n[2], w, dtype=torch.float64)])
         wide = torch.cat([cat(q, Hk * dk), cat(k, Hk * dk), cat(v, H * dv)], dim=1).to(dtype).cuda()      # rows inside wider rows
-        dec = torch.cat([a[0][at[0]: at[0] + n[0]], a[1][at[1]: at[1] + n[1]], torch.ones((n[2],) + tuple(a[0].shape[1:]), dtype=torch.float64)])
+        dec = torch.cat([la[0][at[0]: at[0] + n[0]], la[1][at[1]: at[1] + n[1]], -torch.ones((n[2],) + tuple(a[0].shape[1:]), dtype=torch.float64)])
         ctx = _ctx(n, [2, 0, -1])
         out = torch.full((sum(n), H * dv), 7.0, dtype=torch.float32, device="cuda")
         ops.decay_scan(wide[:, : Hk * dk], wide[:, Hk * dk: 2 * Hk * dk], wide[:, 2 * Hk * dk:], dec.float().cuda().contiguous(),
@@ -322,7 +331,8 @@ def test_decay_scan_in_two_steps(dk, dv, H, Hk, per_channel, dtype):
         at = [at[0] + n[0], at[1] + n[1]]
     for r in range(2):
         g = torch.cat(got[r]).double()
-        assert torch.allclose(g, want[r], atol=1e-3, rtol=2e-4), f"request {r}: max diff {(g - want[r]).abs().max().item():.3g}"
+        assert torch.allclose(g, want[r], atol=2e-5 * want[r].abs().max().item(), rtol=2e-4), \
+            f"request {r}: max diff {(g - want[r]).abs().max().item():.3g} at row {(g - want[r]).abs().max(dim=1).values.argmax().item()}"
     assert state[1].abs().max().item() == 0.0, "a slot that no segment named was written"
     assert state[:, :off].abs().max().item() == 0.0 and state[:, off + need:].abs().max().item() == 0.0
 
@@ -482,12 +492,12 @@ def test_gla_decay_and_the_norm_behind_the_read_out(dtype):
     z = torch.randn(T, C, device="cuda") * 4
     bias = torch.randn(C, device="cuda") * 3
     out = torch.empty_like(z)
-    ops.gla_decay(z, bias, 4.0, out)
+    ops.gla_decay(z, bias, 4.0, out)                                             # the decay's logarithm
     want = torch.sigmoid(z.double() + bias.double()) ** 0.25
-    assert torch.allclose(out.double(), want, atol=1e-6, rtol=1e-5)
+    assert torch.allclose(torch.exp(out.double()), want, atol=1e-6, rtol=1e-5)
     big = torch.tensor([[-200.0, 200.0]], device="cuda")
     ops.gla_decay(big, None, 2.0, big)
-    assert 0.0 <= big[0, 0].item() < 1e-40 and big[0, 1].item() == 1.0          # (e^-100 and 1: no overflow on either side)
+    assert big[0, 0].item() == -100.0 and big[0, 1].item() == 0.0               # (no overflow on either side)
     o = torch.randn(T, H * Dv, device="cuda")
     rows = torch.randn(T, 11 + H * Dv, device="cuda").to(dtype)
     w = torch.rand(Dv, device="cuda") + 0.5
