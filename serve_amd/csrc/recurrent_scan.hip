@@ -20,6 +20,18 @@ __device__ __forceinline__ float rs_softplus(float z) { return fmaxf(z, 0.f) + l
 // ln(sigmoid(z)) without overflow on either side
 __device__ __forceinline__ float rs_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// e^x for x in the range the passes over sixteen tokens use (|x| below 88; a result below the normal range may come
+// out as 0): 2^t with t = x log2(e) rounded, corrected by what the rounding of t lost, r = x log2(e) - t, as
+// 2^t (1 + r ln 2).  A few instructions, and within two units in the last place.
+__device__ __forceinline__ float rs_exp(float x) {
+  const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-8f;
+  const float t = x * L2E;
+  float r = fmaf(x, L2E, -t);
+  r = fmaf(x, L2E_LO, r);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return fmaf(e, r * 0.693147182464599609375f, e);
+}
+
 template <int CTRL>
 __device__ __forceinline__ float rs_dpp(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
@@ -245,32 +257,51 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) S[m][r] = st ? st[state_at(16 * m + 4 * g + r)] : 0.f;
 
-  // the inputs of a pass, in registers: log decays (threads below DKP: one channel each), q, k, v
-  float rla[16], rq[NE], rk[NE], rv[4];
-  auto fetch = [&](int c0) {
-    const int m = min(16, n - c0);
-    if (tid < DKP) {
+  // the inputs of a pass, in registers as they were loaded (nothing is computed on them before their pass, so the
+  // loads of the next pass stay in flight under this one's products): log decays (threads below DKP: one channel
+  // each), q, k, v.  Places outside the segment or the head load a neighbour's value and are masked at use.
+  float rla[16];
+  TQ rq[NE], rk[NE], rv[4];
+  // where a thread's loads lie from the first token of a pass on: 32-bit offsets that change only for a last,
+  // shorter pass (beside a base that is the same for the whole workgroup, a load is then one instruction)
+  unsigned lo[16], qo[NE], ko[NE], vo[4];
+  auto place = [&](int last) {
+    const unsigned c = (unsigned)min(tid, dk - 1);
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const size_t tok = (size_t)(t0 + c0 + t);
-        rla[t] = (t < m && tid < dk) ? (per_channel ? log_decay[(tok * H + h) * (size_t)dk + tid] : log_decay[tok * H + h]) : 0.f;
-      }
+    for (int t = 0; t < 16; ++t) {
+      const unsigned tt = (unsigned)min(t, last);
+      lo[t] = per_channel ? (tt * H) * (unsigned)dk + c : tt * H;
     }
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
-      const int idx = tid + 256 * e, t = idx / DKP, c = idx % DKP;
-      const bool in = t < m && c < dk;
-      const size_t tok = (size_t)(t0 + c0 + t);
-      rq[e] = in ? to_float(q[tok * q_stride + (size_t)hk * dk + c]) * q_scale : 0.f;
-      rk[e] = in ? to_float(k[tok * k_stride + (size_t)hk * dk + c]) : 0.f;
+      const int idx = tid + 256 * e;
+      const unsigned tt = (unsigned)min(idx / DKP, last), cc = (unsigned)min(idx % DKP, dk - 1);
+      qo[e] = tt * (unsigned)q_stride + cc;
+      ko[e] = tt * (unsigned)k_stride + cc;
+    }
+    const unsigned vcol = (unsigned)min(tile * 64 + (tid & 63), dv - 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vo[e] = (unsigned)min((tid + 256 * e) >> 6, last) * (unsigned)v_stride + vcol;
+  };
+  auto fetch = [&](int c0) {
+    const size_t tok = (size_t)(t0 + c0);
+    const float* lb = log_decay + (per_channel ? (tok * H + h) * (size_t)dk : tok * H + h);
+    const TQ* qb = q + tok * q_stride + (size_t)hk * dk;
+    const TQ* kb = k + tok * k_stride + (size_t)hk * dk;
+    const TQ* vb = v + tok * v_stride + (size_t)h * dv;
+    if (tid < DKP) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) rla[t] = lb[lo[t]];
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int idx = tid + 256 * e, t = idx >> 6, c = idx & 63;
-      const int jj = tile * 64 + c;
-      rv[e] = (t < m && jj < dv) ? to_float(v[(size_t)(t0 + c0 + t) * v_stride + (size_t)h * dv + jj]) : 0.f;
+    for (int e = 0; e < NE; ++e) {
+      rq[e] = qb[qo[e]];
+      rk[e] = kb[ko[e]];
     }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) rv[e] = vb[vo[e]];
   };
+  place(min(16, n) - 1);
   fetch(0);
   for (int c0 = 0; c0 < n; c0 += 16) {
     const int m = min(16, n - c0);
@@ -280,29 +311,34 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
       float run = 0.f, b7 = 0.f;
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        run += rla[t];
+        run += (t < m && tid < dk) ? rla[t] : 0.f;
         sb[t][tid] = run;
         if (t == 7) b7 = run;
       }
-      sdec[tid] = expf(run);
+      sdec[tid] = rs_exp(run);
       far = (b7 < -RS_RANGE) || (run - b7 < -RS_RANGE);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int idx = tid + 256 * e;
-      sv[idx >> 6][idx & 63] = rv[e];
+      sv[idx >> 6][idx & 63] = ((idx >> 6) < m && tile * 64 + (idx & 63) < dv) ? to_float(rv[e]) : 0.f;
     }
     const int wide = __syncthreads_or(far);
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
       const int idx = tid + 256 * e, t = idx / DKP, c = idx % DKP;
+      const bool in = t < m && c < dk;
+      const float qv = in ? to_float(rq[e]) * q_scale : 0.f, kv = in ? to_float(rk[e]) : 0.f;
       const float bt = sb[t][c], b7 = sb[7][c], b15 = sb[15][c];
-      sqh[t][c] = rq[e] * expf(bt);
-      skt[t][c] = rk[e] * expf(b15 - bt);
-      sqp[t][c] = wide ? rq[e] : rq[e] * expf(bt - b7);
-      skp[t][c] = wide ? rk[e] : rk[e] * expf(b7 - bt);
+      sqh[t][c] = qv * rs_exp(bt);
+      skt[t][c] = kv * rs_exp(b15 - bt);
+      sqp[t][c] = wide ? qv : qv * rs_exp(bt - b7);
+      skp[t][c] = wide ? kv : kv * rs_exp(b7 - bt);
     }
-    if (c0 + 16 < n) fetch(c0 + 16);             // in flight while the products run
+    if (c0 + 16 < n) {                           // in flight while the products run
+      if (n - (c0 + 16) < 16) place(n - (c0 + 16) - 1);
+      fetch(c0 + 16);
+    }
     __syncthreads();
     // A, the weights of the pass's own tokens
     if (!wide) {
@@ -320,7 +356,7 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
       const int t = tid >> 4, s = tid & 15;
       float a = 0.f;
       if (s <= t)
-        for (int c = 0; c < DKP; ++c) a = fmaf(sqp[t][c] * skp[s][c], expf(sb[t][c] - sb[s][c]), a);
+        for (int c = 0; c < DKP; ++c) a = fmaf(sqp[t][c] * skp[s][c], rs_exp(sb[t][c] - sb[s][c]), a);
       sam[t][s] = a;
     }
     __syncthreads();
@@ -400,7 +436,9 @@ extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dt
       !cu_q || !state_slots || B > 65535 || H > 65535)
     return SA_ERR_ARG;
   const int rpt = scan_rpt(dk), cpt = scan_cpt(dv);
-  if (max_q >= RS_BLOCK_MIN_TOKENS && dk <= RS_BLOCK_MAX_DK && (dtype == SA_F32 || dtype == SA_BF16)) {
+  const long long far_stride = 1LL << 27;         // the passes over sixteen tokens keep 32-bit offsets within a pass
+  if (max_q >= RS_BLOCK_MIN_TOKENS && dk <= RS_BLOCK_MAX_DK && (dtype == SA_F32 || dtype == SA_BF16) &&
+      q_stride < far_stride && k_stride < far_stride && v_stride < far_stride && (long long)H * dk < far_stride) {
     const int rc = dtype == SA_F32
         ? launch_scan_block<float>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
                                    state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream)
@@ -569,39 +607,86 @@ extern "C" int sa_conv_state_update(const void* zx, int dtype, long long zs, int
 //   else:        y = u / sqrt(mean_group(u^2) + eps) * w[i % wn] * silu(g[t, i])
 // g: rows of gate_stride elements in the output's storage type, read from column gate_col on.
 // ---------------------------------------------------------------------------------------------
-// WAVES: how many waves share a group (1: a wave a group, four groups a block; 4: a block a group, for groups of
-// thousands, where a single wave's chain of loads would decide the time of a decode step)
+// WAVES: how many waves share a group (1: a wave a group, four groups a workgroup of 256; 16: a workgroup of 1024 a
+// group, for groups of thousands, where a few waves' chains of loads and divisions would decide the time of a
+// decode step)
 template <typename TA, int WAVES>
-__global__ __launch_bounds__(256) void gated_group_norm_kernel(
+__global__ __launch_bounds__(WAVES == 1 ? 256 : 64 * WAVES) void gated_group_norm_kernel(
     const float* __restrict__ o, const float* __restrict__ skip_x, long long skip_stride,
     const float* __restrict__ skip_d, int dv, const TA* __restrict__ gate, long long gate_stride, int gate_col,
     const float* __restrict__ w, int wn, int group, int gate_first, float eps, TA* __restrict__ y, long long units,
     int n) {
-  __shared__ float part[4];
+  __shared__ float part[WAVES];
   constexpr int LANES = SA_WAVE * WAVES;
   const int lane = threadIdx.x & (LANES - 1);
-  const long long unit = (long long)blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
-  if (unit >= units) return;                    // (whole blocks when WAVES is 4)
+  const long long unit = WAVES == 1 ? (long long)blockIdx.x * 4 + threadIdx.x / SA_WAVE : (long long)blockIdx.x;
+  if (unit >= units) return;                    // (whole workgroups when a workgroup has one group)
   const int groups = n / group;
   const long long t = unit / groups;
   const int i0 = (int)(unit - t * groups) * group;
   const float* orow = o + (size_t)t * n;
   const TA* grow = gate + (size_t)t * gate_stride + gate_col;
+  // a group of up to KEEP LANES values stays in registers between the two passes, and its loads are issued
+  // together; a longer one is read twice
+  constexpr int KEEP = 16;
+  const bool kept = group <= KEEP * LANES;
+  float ku[KEEP], kg[KEEP];
   float ss = 0.f;
-  for (int e = lane; e < group; e += LANES) {
-    const int i = i0 + e;
-    float u = orow[i];
-    if (skip_x) u = fmaf(skip_d[i / dv], skip_x[(size_t)t * skip_stride + i], u);
-    if (gate_first) u *= rs_silu(to_float(grow[i]));
-    ss = fmaf(u, u, ss);
+  if (kept) {
+    float ro[KEEP], rx[KEEP];
+    TA rg[KEEP];
+#pragma unroll
+    for (int x = 0; x < KEEP; ++x) {               // the loads, with nothing between them that waits for one
+      if (x * LANES >= group) break;
+      const int i = i0 + min(lane + x * LANES, group - 1);
+      ro[x] = orow[i];
+      rx[x] = skip_x ? skip_x[(size_t)t * skip_stride + i] : 0.f;
+      rg[x] = grow[i];
+    }
+#pragma unroll
+    for (int x = 0; x < KEEP; ++x) {
+      if (x * LANES >= group) break;
+      const int e = lane + x * LANES, i = i0 + min(e, group - 1);
+      float u = ro[x];
+      if (skip_x) u = fmaf(skip_d[i / dv], rx[x], u);
+      const float g = rs_silu(to_float(rg[x]));
+      if (gate_first) u *= g;
+      if (e >= group) u = 0.f;
+      ku[x] = u;
+      kg[x] = g;
+      ss = fmaf(u, u, ss);
+    }
+  } else {
+    for (int e = lane; e < group; e += LANES) {
+      const int i = i0 + e;
+      float u = orow[i];
+      if (skip_x) u = fmaf(skip_d[i / dv], skip_x[(size_t)t * skip_stride + i], u);
+      if (gate_first) u *= rs_silu(to_float(grow[i]));
+      ss = fmaf(u, u, ss);
+    }
   }
   ss = wave_sum(ss);
   if (WAVES > 1) {
     if ((threadIdx.x & (SA_WAVE - 1)) == 0) part[threadIdx.x / SA_WAVE] = ss;
     __syncthreads();
-    ss = (part[0] + part[1]) + (part[2] + part[3]);
+    ss = 0.f;
+#pragma unroll
+    for (int x = 0; x < WAVES; ++x) ss += part[x];
   }
   const float rs = 1.0f / sqrtf(ss / (float)group + eps);
+  if (kept) {
+#pragma unroll
+    for (int x = 0; x < KEEP; ++x) {
+      if (x * LANES >= group) break;
+      const int e = lane + x * LANES, i = i0 + e;
+      if (e < group) {
+        float out = (ku[x] * rs) * w[i % wn];
+        if (!gate_first) out *= kg[x];
+        y[(size_t)t * n + i] = from_float<TA>(out);
+      }
+    }
+    return;
+  }
   for (int e = lane; e < group; e += LANES) {
     const int i = i0 + e;
     float u = orow[i];
@@ -622,15 +707,15 @@ extern "C" int sa_gated_group_norm(const float* o, const float* skip_x, long lon
   if (!o || !gate || !w || !y || n <= 0 || group <= 0 || n % group || wn <= 0 || dv <= 0 || (skip_x && !skip_d))
     return SA_ERR_ARG;
   const long long units = (long long)T * (n / group);
-  const bool whole = group >= 512;              // a block a group
+  const bool whole = group >= 1024;             // a workgroup a group
   const long long blocks = whole ? units : (units + 3) / 4;
   if (blocks > 0x7fffffffLL) return SA_ERR_ARG;
-  dim3 grid((unsigned)blocks), block(256);
+  dim3 grid((unsigned)blocks), block(whole ? 1024 : 256);
 #define GO(TA, W) hipLaunchKernelGGL((gated_group_norm_kernel<TA, W>), grid, block, 0, stream, o, skip_x, skip_stride, skip_d, dv, (const TA*)gate, gate_stride, gate_col, w, wn, group, gate_first, eps, (TA*)y, units, n)
   if (dtype == SA_F32) {
-    if (whole) GO(float, 4); else GO(float, 1);
+    if (whole) GO(float, 16); else GO(float, 1);
   } else if (dtype == SA_BF16) {
-    if (whole) GO(bf16_t, 4); else GO(bf16_t, 1);
+    if (whole) GO(bf16_t, 16); else GO(bf16_t, 1);
   } else {
     return SA_ERR_UNSUPPORTED;
   }

@@ -19,7 +19,7 @@ __global__ __launch_bounds__(256) void stream_add_kernel(float* __restrict__ x, 
                                                          size_t part_stride, const float* __restrict__ vec,
                                                          TA* __restrict__ h, int d) {
   const size_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += blockDim.x * gridDim.y) {
     const size_t at = t * d + i;
     float v = x[at];
     if (y) v += parts_at(y, parts, part_stride, at);
@@ -33,7 +33,8 @@ template <typename TA>
 static int launch_stream_add(float* x, const void* y, int y_dtype, int parts, const float* vec, void* h, int T, int d,
                              hipStream_t stream) {
   const size_t ps = (size_t)T * d;
-  dim3 grid(T), block(256);
+  // a step of few rows: a value a thread, so that a row's loads are not a chain in one workgroup
+  dim3 grid(T, T <= 64 ? (unsigned)((d + 255) / 256) : 1u), block(256);
   if (!y || y_dtype == SA_F32)
     hipLaunchKernelGGL((stream_add_kernel<TA, float>), grid, block, 0, stream, x, (const float*)y, parts, ps, vec, (TA*)h, d);
   else if (y_dtype == SA_BF16)
@@ -58,10 +59,11 @@ extern "C" int sa_stream_add(float* x, const void* y, int y_dtype, int parts, co
 
 // ---------------------------------------------------------------------------------------------
 // Two mixers side by side: out[t] = ca N(a[t]) wa + cb N(b[t]) wb,  N(y) = y / sqrt(mean(y^2) + eps), fp32 out [T, d].
-// a and b: [T, d] or fp32 [parts, T, d] each.  One workgroup a row; a thread keeps up to VMAX values of each.
+// a and b: [T, d] or fp32 [parts, T, d] each.  One workgroup a row; a thread keeps up to VMAX values of each.  A step
+// of few rows takes workgroups of 1024 threads: a row's partial sums are then a few loads a thread, not a chain.
 // ---------------------------------------------------------------------------------------------
 template <typename TDA, typename TDB>
-__global__ __launch_bounds__(256) void dual_norm_mix_kernel(const TDA* __restrict__ a, int parts_a,
+__global__ __launch_bounds__(1024) void dual_norm_mix_kernel(const TDA* __restrict__ a, int parts_a,
                                                             const TDB* __restrict__ b, int parts_b,
                                                             size_t part_stride, const float* __restrict__ wa,
                                                             const float* __restrict__ wb, float ca, float cb, float eps,
@@ -112,7 +114,7 @@ extern "C" int sa_dual_norm_mix(const void* a, int a_dtype, int parts_a, const v
       (parts_b > 1 && b_dtype != SA_F32))
     return SA_ERR_ARG;
   const size_t ps = (size_t)T * d;
-  dim3 grid(T), block(256);
+  dim3 grid(T), block(T <= 64 && d >= 1024 ? 1024 : 256);
 #define GO(TDA, TDB)                                                                                             \
   hipLaunchKernelGGL((dual_norm_mix_kernel<TDA, TDB>), grid, block, 0, stream, (const TDA*)a, parts_a, (const TDB*)b, \
                      parts_b, ps, wa, wb, ca, cb, eps, out, d)
