@@ -257,7 +257,7 @@ extern "C" int sa_qk_norm_kv_write(const void* qkv, int row_stride, void* q_out,
 // EXACT: sincosf of the float32 path; else the reduced-argument hardware sine and cosine.
 // ---------------------------------------------------------------------------------------------
 template <typename TA, bool EXACT>
-__global__ __launch_bounds__(256) void row_norm_rope_kv_write_kernel(
+__global__ __launch_bounds__(1024) void row_norm_rope_kv_write_kernel(
     const TA* __restrict__ qkv, long long row_stride, TA* __restrict__ q_out, const int* __restrict__ positions,
     const int* __restrict__ slot, TA* __restrict__ k_pages, TA* __restrict__ v_pages, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, const float* __restrict__ freq, int rot, int T, int Hq, int Hk, int D,
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(256) void row_norm_rope_kv_write_kernel(
     return;
   }
   if (!slot) return;
-  const long long idx = (long long)(blockIdx.x - T) * 256 + threadIdx.x;
+  const long long idx = (long long)(blockIdx.x - T) * blockDim.x + threadIdx.x;
   if (idx >= (long long)T * Hk * Dp) return;
   const int t = (int)(idx % T);
   const int gi = (int)(idx / T);
@@ -336,9 +336,11 @@ extern "C" int sa_row_norm_rope_kv_write(const void* qkv, long long row_stride, 
   if (row_stride < (long long)Hq * D + (long long)Hk * (D + Dv) || (slot && (!k_pages || !v_pages)) || rot < 0 || rot % 2 ||
       rot > D || (rot > 0 && !freq))
     return SA_ERR_ARG;
-  const long long v_blocks = slot ? ((long long)T * Hk * Dp + 255) / 256 : 0;
+  // a step of few tokens takes workgroups of 1024: a token's row is then two or three values a thread
+  const int threads = T <= 64 ? 1024 : 256;
+  const long long v_blocks = slot ? ((long long)T * Hk * Dp + threads - 1) / threads : 0;
   if ((long long)T + v_blocks > 0x7fffffffLL) return SA_ERR_ARG;
-  dim3 grid((unsigned)(T + v_blocks)), block(256);
+  dim3 grid((unsigned)(T + v_blocks)), block(threads);
   if (act_dtype == SA_F32)
     hipLaunchKernelGGL((row_norm_rope_kv_write_kernel<float, true>), grid, block, 0, stream, (const float*)qkv, row_stride,
                        (float*)q_out, positions, slot, (float*)k_pages, (float*)v_pages, wq, wk, eps, freq, rot, T, Hq, Hk,
