@@ -218,13 +218,18 @@ static void launch_scan_r(int rpt, int cpt, const void* q, const void* k, const 
 // ---------------------------------------------------------------------------------------------
 typedef float rs_f4 __attribute__((ext_vector_type(4)));
 #define RS_RANGE 80.f
+// what a launch of the kernel does: whole segments from the requests' states; or, where long segments are cut into
+// pieces that run side by side, first every piece from zeros for the state that its tokens add, then (after the chain
+// through the pieces) every piece from the state it truly starts from
+enum { RS_WHOLE = 0, RS_PIECE_STATES = 1, RS_PIECE_OUTPUTS = 2 };
 
 template <typename TQ, int NT>
 __global__ __launch_bounds__(256) void decay_scan_block_kernel(
     const TQ* __restrict__ q, const TQ* __restrict__ k, const TQ* __restrict__ v, long long q_stride,
     long long k_stride, long long v_stride, const float* __restrict__ log_decay, int per_channel, float q_scale,
     float* __restrict__ state, long long state_stride, const int* __restrict__ cu_q,
-    const int* __restrict__ state_slots, float* __restrict__ o, int H, int Hk, int dk, int dv, int RPT, int CPT) {
+    const int* __restrict__ state_slots, float* __restrict__ o, int H, int Hk, int dk, int dv, int RPT, int CPT,
+    int mode, int piece, int pieces, float* __restrict__ scratch, long long scratch_stride, long long scratch_decays) {
   constexpr int DKP = 16 * NT;                   // the key channels, padded
   constexpr int ST = DKP + 4;                    // row stride in LDS: 4 (or 20) mod 32 banks, and rows stay 16-byte aligned
   constexpr int NE = NT;                         // q / k elements of a pass per thread: 16 DKP / 256
@@ -238,11 +243,14 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
   __shared__ float sap[4][16][17];
   __shared__ float sam[16][20];
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, j = lane & 15;
-  const int tile = blockIdx.x, h = blockIdx.y, seg = blockIdx.z;
+  const int tile = blockIdx.x, h = blockIdx.y, seg = blockIdx.z / pieces, pj = blockIdx.z - seg * pieces;
   const int hk = h / (H / Hk);
   const int slot = state_slots[seg];
-  const int t0 = cu_q[seg], n = cu_q[seg + 1] - t0;
+  const int whole = cu_q[seg + 1] - cu_q[seg];   // the segment; this workgroup's piece of it: n tokens from t0
+  const int t0 = cu_q[seg] + pj * piece, n = min(piece, cu_q[seg + 1] - t0);
   if (n <= 0) return;
+  const bool split = whole > piece;              // the segment has several pieces: their states go through `scratch`
+  if (mode == RS_PIECE_STATES && !split) return;
   const int col = tile * 64 + w * 16 + j;        // this lane's column of S and o
   const int seq_tiles = (dv + 16 * CPT - 1) / (16 * CPT);
   // where the token-by-token kernel keeps (row, col) of head h
@@ -250,12 +258,14 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
     return (((size_t)h * seq_tiles + col / (16 * CPT)) * RPT + row % RPT) * (size_t)(256 * CPT) +
            (size_t)(((col / CPT) % 16) * 16 + row / RPT) * CPT + col % CPT;
   };
-  float* st = slot >= 0 && col < dv ? state + (size_t)slot * state_stride : nullptr;
+  float* const mine = scratch + (size_t)blockIdx.z * scratch_stride;      // this piece's row of the scratch
+  float* st = col >= dv ? nullptr : (split ? mine : (slot >= 0 ? state + (size_t)slot * state_stride : nullptr));
   rs_f4 S[NT];
 #pragma unroll
   for (int m = 0; m < NT; ++m)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) S[m][r] = st ? st[state_at(16 * m + 4 * g + r)] : 0.f;
+    for (int r = 0; r < 4; ++r) S[m][r] = (st && mode != RS_PIECE_STATES) ? st[state_at(16 * m + 4 * g + r)] : 0.f;
+  float btotal = 0.f;                            // (threads below DKP) the piece's sum of a channel's log decays
 
   // the inputs of a pass, in registers as they were loaded (nothing is computed on them before their pass, so the
   // loads of the next pass stay in flight under this one's products): log decays (threads below DKP: one channel
@@ -316,6 +326,7 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
         if (t == 7) b7 = run;
       }
       sdec[tid] = rs_exp(run);
+      btotal += run;
       far = (b7 < -RS_RANGE) || (run - b7 < -RS_RANGE);
     }
 #pragma unroll
@@ -330,10 +341,12 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
       const bool in = t < m && c < dk;
       const float qv = in ? to_float(rq[e]) * q_scale : 0.f, kv = in ? to_float(rk[e]) : 0.f;
       const float bt = sb[t][c], b7 = sb[7][c], b15 = sb[15][c];
-      sqh[t][c] = qv * rs_exp(bt);
       skt[t][c] = kv * rs_exp(b15 - bt);
-      sqp[t][c] = wide ? qv : qv * rs_exp(bt - b7);
-      skp[t][c] = wide ? kv : kv * rs_exp(b7 - bt);
+      if (mode != RS_PIECE_STATES) {
+        sqh[t][c] = qv * rs_exp(bt);
+        sqp[t][c] = wide ? qv : qv * rs_exp(bt - b7);
+        skp[t][c] = wide ? kv : kv * rs_exp(b7 - bt);
+      }
     }
     if (c0 + 16 < n) {                           // in flight while the products run
       if (n - (c0 + 16) < 16) place(n - (c0 + 16) - 1);
@@ -341,7 +354,8 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
     }
     __syncthreads();
     // A, the weights of the pass's own tokens
-    if (!wide) {
+    if (mode == RS_PIECE_STATES) {
+    } else if (!wide) {
       rs_f4 acc = {0.f, 0.f, 0.f, 0.f};
       const int cb = w * 4 * NT;                 // each wave a quarter of the channels
 #pragma unroll
@@ -364,19 +378,21 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
     float vb[4];
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) vb[s4] = sv[4 * s4 + g][w * 16 + j];
-    rs_f4 oc = {0.f, 0.f, 0.f, 0.f};
+    if (mode != RS_PIECE_STATES) {
+      rs_f4 oc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int mt = 0; mt < NT; ++mt) {
-      const rs_f4 a4 = *reinterpret_cast<const rs_f4*>(&sqh[j][16 * mt + 4 * g]);
+      for (int mt = 0; mt < NT; ++mt) {
+        const rs_f4 a4 = *reinterpret_cast<const rs_f4*>(&sqh[j][16 * mt + 4 * g]);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], S[mt][r], oc, 0, 0, 0);
-    }
+        for (int r = 0; r < 4; ++r) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[r], S[mt][r], oc, 0, 0, 0);
+      }
 #pragma unroll
-    for (int s4 = 0; s4 < 4; ++s4) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(sam[j][4 * s4 + g], vb[s4], oc, 0, 0, 0);
-    if (col < dv) {
+      for (int s4 = 0; s4 < 4; ++s4) oc = __builtin_amdgcn_mfma_f32_16x16x4f32(sam[j][4 * s4 + g], vb[s4], oc, 0, 0, 0);
+      if (col < dv) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (4 * g + r < m) o[((size_t)(t0 + c0 + 4 * g + r) * H + h) * dv + col] = oc[r];
+        for (int r = 0; r < 4; ++r)
+          if (4 * g + r < m) o[((size_t)(t0 + c0 + 4 * g + r) * H + h) * dv + col] = oc[r];
+      }
     }
     // ... and the state after the pass
 #pragma unroll
@@ -390,21 +406,57 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
       S[mt] = sm;
     }
   }
-  if (st) {
+  // a whole segment leaves its state with the request; a piece leaves what its own tokens add to a state (and by how
+  // much they shrink one) in its row of the scratch, and nothing after the pass that starts from the true state
+  if (st && (mode == RS_PIECE_STATES || !split)) {
 #pragma unroll
     for (int m = 0; m < NT; ++m)
 #pragma unroll
       for (int r = 0; r < 4; ++r) st[state_at(16 * m + 4 * g + r)] = S[m][r];
   }
+  if (mode == RS_PIECE_STATES && tile == 0 && tid < DKP) mine[scratch_decays + (size_t)h * DKP + tid] = rs_exp(btotal);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Between the two passes over the pieces of long segments: from the request's state (or zeros) S, piece after piece,
+// the piece's row takes S, the state it starts from, and S <- D S + (what the piece's tokens add), D the piece's
+// decay of the row's key channel; the state after the last piece goes to the request.  A thread per float of a
+// state row (the token-by-token kernel's layout: index -> row as there); grid (ceil(floats / 256), B).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void decay_scan_chain_kernel(float* __restrict__ state, long long state_stride,
+                                                               const int* __restrict__ cu_q,
+                                                               const int* __restrict__ state_slots,
+                                                               float* __restrict__ scratch, long long scratch_stride,
+                                                               long long scratch_decays, int floats, int piece,
+                                                               int pieces, int RPT, int CPT, int DKP, int tiles) {
+  const int seg = blockIdx.y;
+  const int whole = cu_q[seg + 1] - cu_q[seg];
+  const int at = blockIdx.x * 256 + threadIdx.x;
+  if (whole <= piece || at >= floats) return;
+  const int count = (whole + piece - 1) / piece;
+  // at = ((h tiles + tile) RPT + ii) 256 CPT + thread CPT + cc, thread = 16 (column group) + r: row r RPT + ii
+  const int per = 256 * CPT;
+  const int hi = at / per, thread = (at - hi * per) / CPT;
+  const int h = hi / (tiles * RPT), row = (thread & 15) * RPT + hi % RPT;
+  const int slot = state_slots[seg];
+  float S = slot >= 0 ? state[(size_t)slot * state_stride + at] : 0.f;
+  for (int pj = 0; pj < count; ++pj) {
+    float* mine = scratch + (size_t)(seg * pieces + pj) * scratch_stride;
+    const float add = mine[at], D = mine[scratch_decays + (size_t)h * DKP + row];
+    mine[at] = S;
+    S = fmaf(D, S, add);
+  }
+  if (slot >= 0) state[(size_t)slot * state_stride + at] = S;
 }
 
 template <typename TQ>
 static int launch_scan_block(int rpt, int cpt, const void* q, const void* k, const void* v, long long qs, long long ks,
                              long long vs, const float* decay, int per_channel, float q_scale, float* state,
                              long long state_stride, const int* cu_q, const int* slots, float* o, int B, int H, int Hk,
-                             int dk, int dv, hipStream_t stream) {
-  dim3 grid((dv + 63) / 64, H, B), block(256);
-#define GO(N) hipLaunchKernelGGL((decay_scan_block_kernel<TQ, N>), grid, block, 0, stream, (const TQ*)q, (const TQ*)k, (const TQ*)v, qs, ks, vs, decay, per_channel, q_scale, state, state_stride, cu_q, slots, o, H, Hk, dk, dv, rpt, cpt)
+                             int dk, int dv, int mode, int piece, int pieces, float* scratch, long long scratch_stride,
+                             long long scratch_decays, hipStream_t stream) {
+  dim3 grid((dv + 63) / 64, H, B * pieces), block(256);
+#define GO(N) hipLaunchKernelGGL((decay_scan_block_kernel<TQ, N>), grid, block, 0, stream, (const TQ*)q, (const TQ*)k, (const TQ*)v, qs, ks, vs, decay, per_channel, q_scale, state, state_stride, cu_q, slots, o, H, Hk, dk, dv, rpt, cpt, mode, piece, pieces, scratch, scratch_stride, scratch_decays)
   switch (rpt) {
     case 1: GO(1); break;
     case 2: GO(2); break;
@@ -430,7 +482,7 @@ extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dt
                              long long k_stride, long long v_stride, const float* decay, int per_channel,
                              float q_scale, float* state, long long state_stride, const int* cu_q,
                              const int* state_slots, float* o, int B, int H, int Hk, int dk, int dv, int max_q,
-                             hipStream_t stream) {
+                             int piece, float* scratch, long long scratch_stride, hipStream_t stream) {
   if (B <= 0) return 0;
   if (H <= 0 || Hk <= 0 || H % Hk || dk <= 0 || dk > 256 || dv <= 0 || !q || !k || !v || !decay || !state || !o ||
       !cu_q || !state_slots || B > 65535 || H > 65535)
@@ -439,13 +491,36 @@ extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dt
   const long long far_stride = 1LL << 27;         // the passes over sixteen tokens keep 32-bit offsets within a pass
   if (max_q >= RS_BLOCK_MIN_TOKENS && dk <= RS_BLOCK_MAX_DK && (dtype == SA_F32 || dtype == SA_BF16) &&
       q_stride < far_stride && k_stride < far_stride && v_stride < far_stride && (long long)H * dk < far_stride) {
-    const int rc = dtype == SA_F32
-        ? launch_scan_block<float>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
-                                   state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream)
-        : launch_scan_block<bf16_t>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
-                                    state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, stream);
-    if (rc) return rc;
-    SA_LAUNCH_CHECK();
+    // piece > 0: segments longer than `piece` tokens (a multiple of 16) run as pieces side by side; scratch: fp32 rows
+    // of scratch_stride >= state floats + H 16 rpt floats, one per (segment, piece), B ceil(max_q / piece) of them
+    const long long floats = sa_decay_scan_state_floats(H, dk, dv);
+    int pieces = 1;
+    if (piece > 0 && max_q > piece) {
+      if (piece % 16 || !scratch || scratch_stride < floats + (long long)H * 16 * rpt) return SA_ERR_ARG;
+      pieces = (max_q + piece - 1) / piece;
+    } else {
+      piece = 0x7fffff00;
+    }
+    if ((long long)B * pieces > 65535) return SA_ERR_ARG;
+    const int modes[2] = {pieces > 1 ? RS_PIECE_STATES : RS_WHOLE, RS_PIECE_OUTPUTS};
+    for (int pass = 0; pass < (pieces > 1 ? 2 : 1); ++pass) {
+      const int rc = dtype == SA_F32
+          ? launch_scan_block<float>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
+                                     state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, modes[pass], piece, pieces,
+                                     scratch, scratch_stride, floats, stream)
+          : launch_scan_block<bf16_t>(rpt, cpt, q, k, v, q_stride, k_stride, v_stride, decay, per_channel, q_scale, state,
+                                      state_stride, cu_q, state_slots, o, B, H, Hk, dk, dv, modes[pass], piece, pieces,
+                                      scratch, scratch_stride, floats, stream);
+      if (rc) return rc;
+      SA_LAUNCH_CHECK();
+      if (pieces > 1 && pass == 0) {
+        const int tiles = (dv + 16 * cpt - 1) / (16 * cpt);
+        hipLaunchKernelGGL(decay_scan_chain_kernel, dim3((unsigned)((floats + 255) / 256), B), dim3(256), 0, stream, state,
+                           state_stride, cu_q, state_slots, scratch, scratch_stride, floats, (int)floats, piece, pieces,
+                           rpt, cpt, 16 * rpt, tiles);
+        SA_LAUNCH_CHECK();
+      }
+    }
     return 0;
   }
   if (dtype == SA_F32)

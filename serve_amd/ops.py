@@ -742,6 +742,16 @@ def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, col: int, tokens: torch.
 SCAN_MAX_DIM = 256
 SCAN_MAX_TAPS = 16
 SCAN_BLOCK_MIN_TOKENS = 6        # csrc/recurrent_scan.hip: RS_BLOCK_MIN_TOKENS
+SCAN_PIECE_MIN = 64              # the shortest piece that a long segment is cut into
+SCAN_PIECE_GROUPS = 512          # workgroups that a step's recurrence should at least have
+
+
+def _pow2_rows(dk: int) -> int:
+    """16 x a power of two that holds dk rows, over 16: the recurrence kernels' padding of the key size."""
+    rpt = 1
+    while 16 * rpt < dk:
+        rpt *= 2
+    return rpt
 
 
 def decay_scan_state_floats(heads: int, dk: int, dv: int) -> int:
@@ -749,9 +759,7 @@ def decay_scan_state_floats(heads: int, dk: int, dv: int) -> int:
     layout, rows padded to 16 x a power of two and columns to whole tiles (csrc/recurrent_scan.hip)."""
     if not (heads > 0 and 0 < dk <= SCAN_MAX_DIM and dv > 0):
         raise KernelError(f"decay_scan takes key sizes up to {SCAN_MAX_DIM}; got heads {heads}, dk {dk}, dv {dv}")
-    rpt = 1
-    while 16 * rpt < dk:
-        rpt *= 2
+    rpt = _pow2_rows(dk)
     cpt = 4 if dv >= 64 else (2 if dv >= 32 else 1)
     tiles = -(-dv // (16 * cpt))
     return heads * tiles * rpt * 256 * cpt
@@ -764,13 +772,14 @@ def _rows(t: torch.Tensor, T: int, width: int, name: str) -> None:
 
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
                state_offset: int, ctx, out: torch.Tensor, heads: int, qk_heads: int, dk: int, dv: int,
-               q_scale: float = 1.0) -> torch.Tensor:
+               q_scale: float = 1.0, piece_ok: bool = True) -> torch.Tensor:
     """Per segment of the step and head h, from the request's state S (fp32, zeros for a new request), token by token:
     S = diag(a) S + k v^T, out = S^T (q_scale q).  q, k: rows [T, >= qk_heads dk] (views with a row stride are fine;
     head h reads q/k head h // (heads / qk_heads)); v rows [T, >= heads dv]; all three of one dtype.  decay: ln a, fp32
     [T, heads, dk] (one per key channel) or [T, heads] (one per head).  A step whose longest segment has
     `SCAN_BLOCK_MIN_TOKENS` tokens or more takes sixteen tokens a pass on the matrix cores (keys up to 128 wide),
-    any other goes token by token.  state fp32 [slots, row]: the matrices live at
+    any other goes token by token; long segments of a step that would leave most of the chip idle are cut into pieces
+    that run side by side (`piece_ok` False: never).  state fp32 [slots, row]: the matrices live at
     `state_offset` of a request's row (ctx.state_slots, -1: none) in the kernel's own layout
     (`decay_scan_state_floats` floats).  out fp32 [T, heads dv]."""
     T, B = ctx.num_tokens, ctx.num_segments
@@ -792,11 +801,27 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
     _i32(ctx.state_slots, B, "state_slots")
     lib = load_library("recurrent_scan")
     LL = ctypes.c_longlong
+    max_q = int(getattr(ctx, "max_q_len", 0) or T)
+    # a step of few long segments has too few (segment, head, 64 columns) for the chip: its segments are cut into
+    # pieces that run side by side (each piece's own contribution to the state first, a chain through them, then the
+    # pieces again from their true states), through a scratch row per piece
+    piece, scratch = 0, None
+    groups = B * heads * -(-dv // 64)
+    if max_q >= 2 * SCAN_PIECE_MIN and groups < SCAN_PIECE_GROUPS and dk <= 128 and piece_ok:
+        want = -(-SCAN_PIECE_GROUPS // groups)
+        piece = max(SCAN_PIECE_MIN, -(-(-(-max_q // want)) // 16) * 16)
+        if max_q > piece:
+            rows = B * -(-max_q // piece)
+            scratch = torch.zeros((rows, need + heads * 16 * _pow2_rows(dk)),
+                                  dtype=torch.float32, device=out.device)
+        else:
+            piece = 0
     _ret(lib.sa_decay_scan(_ptr(q), _ptr(k), _ptr(v), c_int(_code(q)), LL(q.stride(0)), LL(k.stride(0)), LL(v.stride(0)),
                            _ptr(decay), c_int(1 if per_channel else 0), c_float(q_scale),
                            c_void_p(state.data_ptr() + 4 * state_offset), LL(state.stride(0)), _ptr(ctx.cu_q),
                            _ptr(ctx.state_slots), _ptr(out), c_int(B), c_int(heads), c_int(qk_heads), c_int(dk), c_int(dv),
-                           c_int(int(getattr(ctx, "max_q_len", 0) or T)), _stream()), "decay_scan")
+                           c_int(max_q), c_int(piece), _ptr(scratch), LL(scratch.stride(0) if scratch is not None else 0),
+                           _stream()), "decay_scan")
     return out
 
 

@@ -280,7 +280,9 @@ def _ctx(lens, slots):
 
 
 # steps of two requests and a segment of nobody's: short ones go token by token, the others sixteen tokens a pass
-SCAN_STEPS = {"short": [[4, 1, 3], [1, 5, 2]], "mid": [[9, 1, 3], [1, 21, 2]], "long": [[33, 1, 16], [1, 64, 7], [47, 3, 1]]}
+# (and the longest are cut into pieces that run side by side, with a chain of states between two passes)
+SCAN_STEPS = {"short": [[4, 1, 3], [1, 5, 2]], "mid": [[9, 1, 3], [1, 21, 2]], "long": [[33, 1, 16], [1, 64, 7], [47, 3, 1]],
+              "pieces": [[300, 1, 20], [1, 415, 7], [130, 3, 129]]}
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
