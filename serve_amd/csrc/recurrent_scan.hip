@@ -15,13 +15,7 @@
 
 #define RS_MAX_TAPS 16
 
-__device__ __forceinline__ float rs_silu(float z) { return z / (1.f + expf(-z)); }
-__device__ __forceinline__ float rs_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
-// ln(sigmoid(z)) without overflow on either side
-__device__ __forceinline__ float rs_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
-
-// e^x for x in the range the passes over sixteen tokens use (|x| below 88; a result below the normal range may come
-// out as 0): 2^t with t = x log2(e) rounded, corrected by what the rounding of t lost, r = x log2(e) - t, as
+// e^x in a few instructions (a result below the normal range may come out as 0, one above it as infinity): 2^t with t = x log2(e) rounded, corrected by what the rounding of t lost, r = x log2(e) - t, as
 // 2^t (1 + r ln 2).  A few instructions, and within two units in the last place.
 __device__ __forceinline__ float rs_exp(float x) {
   const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-8f;
@@ -31,6 +25,13 @@ __device__ __forceinline__ float rs_exp(float x) {
   const float e = __builtin_amdgcn_exp2f(t);
   return fmaf(e, r * 0.693147182464599609375f, e);
 }
+
+// z sigmoid(z) with that exponential and the hardware's reciprocal: within a few units in the last place
+// (the exponent is kept below the overflow: beyond 80 the result is z e^z, which is nothing, either way)
+__device__ __forceinline__ float rs_silu(float z) { return z * __builtin_amdgcn_rcpf(1.f + rs_exp(fminf(-z, 80.f))); }
+__device__ __forceinline__ float rs_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+// ln(sigmoid(z)) without overflow on either side
+__device__ __forceinline__ float rs_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 template <int CTRL>
 __device__ __forceinline__ float rs_dpp(float v) {
@@ -565,42 +566,54 @@ extern "C" int sa_gla_decay(const float* z, const float* bias, float tau, float*
 // (w [C, taps], the last column on the current token, bias b; inputs before the segment come from the request's state
 // row at conv_off, [taps - 1, C] oldest first, or are zeros where the segment has no request) and silu -> xbc fp32 [T, C].
 // Per token and head: dt = softplus(dtraw + dt_bias), the decay's logarithm -exp(A_log) dt -> decay [T, H]; v = dt x -> fp32 [T, H P].
-// grid (T, ceil((C + H) / 256)).
+// grid (T, or ceil(T / 8) from 257 tokens on; ceil((C + H) / 256)).
 // ---------------------------------------------------------------------------------------------
+#define RS_PREP_TOKENS 8
 template <typename TA>
 __global__ __launch_bounds__(256) void ssm_prepare_kernel(
     const TA* __restrict__ zx, long long zs, int col0, const float* __restrict__ conv_w,
     const float* __restrict__ conv_b, const float* __restrict__ state, long long state_stride, long long conv_off,
     const float* __restrict__ dtraw, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     const int* __restrict__ seg_of_token, const int* __restrict__ cu_q, const int* __restrict__ state_slots,
-    float* __restrict__ xbc, float* __restrict__ vout, float* __restrict__ decay, int H, int P, int C, int taps) {
-  const int t = blockIdx.x;
+    float* __restrict__ xbc, float* __restrict__ vout, float* __restrict__ decay, int T, int H, int P, int C, int taps, int per) {
+  // `per` tokens a workgroup (in a prompt a token's work for a channel is too little to pay for a workgroup's start);
+  // the step sizes of the heads that the workgroup's channels belong to are made once a head and token
+  __shared__ float sdt[RS_PREP_TOKENS][260];
   const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c_first = blockIdx.y * 256;
+  const int t_end = min(T, ((int)blockIdx.x + 1) * per);
+  const int h_first = c_first / P;
+  if (c_first < H * P) {
+    const int nh = min(c_first + 255, H * P - 1) / P - h_first + 1;
+    for (int i = threadIdx.x; i < nh * per; i += 256) {
+      const int tt = i / nh, hh = i - tt * nh, t = blockIdx.x * per + tt;
+      if (t < t_end) sdt[tt][hh] = rs_softplus(dtraw[(size_t)t * H + h_first + hh] + dt_bias[h_first + hh]);
+    }
+    __syncthreads();
+  }
   if (c >= C + H) return;
-  if (c >= C) {
-    const int h = c - C;
-    const float dt = rs_softplus(dtraw[(size_t)t * H + h] + dt_bias[h]);
-    decay[(size_t)t * H + h] = -expf(A_log[h]) * dt;
-    return;
-  }
-  const int seg = seg_of_token[t];
-  const int t0 = cu_q[seg];
-  const int slot = state_slots[seg];
-  const float* cs = slot >= 0 ? state + (size_t)slot * state_stride + conv_off : nullptr;
-  float acc = conv_b ? conv_b[c] : 0.f;
-  for (int j = 0; j < taps; ++j) {
-    const int tp = t - (taps - 1 - j);
-    float xv;
-    if (tp >= t0) xv = to_float(zx[(size_t)tp * zs + col0 + c]);
-    else xv = cs ? cs[(size_t)(taps - 1 + tp - t0) * C + c] : 0.f;
-    acc = fmaf(conv_w[(size_t)c * taps + j], xv, acc);
-  }
-  const float y = rs_silu(acc);
-  xbc[(size_t)t * C + c] = y;
-  if (c < H * P) {
-    const int h = c / P;
-    const float dt = rs_softplus(dtraw[(size_t)t * H + h] + dt_bias[h]);
-    vout[(size_t)t * H * P + c] = dt * y;
+  for (int t = blockIdx.x * per; t < t_end; ++t) {
+    if (c >= C) {
+      const int h = c - C;
+      const float dt = rs_softplus(dtraw[(size_t)t * H + h] + dt_bias[h]);
+      decay[(size_t)t * H + h] = -expf(A_log[h]) * dt;
+      continue;
+    }
+    const int seg = seg_of_token[t];
+    const int t0 = cu_q[seg];
+    const int slot = state_slots[seg];
+    const float* cs = slot >= 0 ? state + (size_t)slot * state_stride + conv_off : nullptr;
+    float acc = conv_b ? conv_b[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int tp = t - (taps - 1 - j);
+      float xv;
+      if (tp >= t0) xv = to_float(zx[(size_t)tp * zs + col0 + c]);
+      else xv = cs ? cs[(size_t)(taps - 1 + tp - t0) * C + c] : 0.f;
+      acc = fmaf(conv_w[(size_t)c * taps + j], xv, acc);
+    }
+    const float y = rs_silu(acc);
+    xbc[(size_t)t * C + c] = y;
+    if (c < H * P) vout[(size_t)t * H * P + c] = sdt[t - blockIdx.x * per][c / P - h_first] * y;
   }
 }
 
@@ -613,15 +626,16 @@ extern "C" int sa_ssm_prepare(const void* zx, int dtype, long long zs, int col0,
   if (!zx || !conv_w || !state || !dtraw || !A_log || !dt_bias || !xbc || !vout || !decay || H <= 0 || P <= 0 ||
       C < H * P || taps < 1 || taps > RS_MAX_TAPS || (C + H + 255) / 256 > 65535)
     return SA_ERR_ARG;
-  dim3 grid(T, (C + H + 255) / 256), block(256);
+  const int per = T > 256 ? RS_PREP_TOKENS : 1;
+  dim3 grid((T + per - 1) / per, (C + H + 255) / 256), block(256);
   if (dtype == SA_F32)
     hipLaunchKernelGGL(ssm_prepare_kernel<float>, grid, block, 0, stream, (const float*)zx, zs, col0, conv_w, conv_b,
                        state, state_stride, conv_off, dtraw, A_log, dt_bias, seg_of_token, cu_q, state_slots, xbc, vout,
-                       decay, H, P, C, taps);
+                       decay, T, H, P, C, taps, per);
   else if (dtype == SA_BF16)
     hipLaunchKernelGGL(ssm_prepare_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)zx, zs, col0, conv_w, conv_b,
                        state, state_stride, conv_off, dtraw, A_log, dt_bias, seg_of_token, cu_q, state_slots, xbc, vout,
-                       decay, H, P, C, taps);
+                       decay, T, H, P, C, taps, per);
   else
     return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();
