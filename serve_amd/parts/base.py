@@ -215,3 +215,8 @@ class PositionPart(Part):
     def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], positions: torch.Tensor) -> None:
         """Encode in place: q [T, Hq, D] and k [T, Hk, D] (views into the projected rows; k is
         None for a mixer that reads another layer's cache), positions int32 [T]."""
+
+
+# the name under which a layer leaves, on the step's context (`ctx.shared`), (activations, the norm that made them)
+# for the next layer: the norm that layer begins with, applied at the end of this layer's own last kernel
+NORMED_STREAM = "normed_stream"

@@ -21,7 +21,7 @@ import torch
 
 from .. import ops
 from ..registry import register_part
-from .base import LayerCache, ParamRequest, Part, Runtime
+from .base import NORMED_STREAM, LayerCache, ParamRequest, Part, Runtime
 
 
 class ScaledOutputNorm(Part):
@@ -117,7 +117,6 @@ class PostNormResidual:
         return None
 
 
-NORMED_STREAM = "normed_stream"     # (activations, the norm that made them) from one layer for the next, on the step's context
 
 
 class SandwichResidual:

@@ -12,7 +12,7 @@ import torch
 from .. import ops, trace
 from ..config.spec import PartSpec
 from ..registry import get_part, register_part
-from .base import (LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime, StepCost, TokenCacheRequest,
+from .base import (NORMED_STREAM, LayerCache, ParamRequest, Part, PositionPart, Rotary, Runtime, StepCost, TokenCacheRequest,
                    kv_cache_request)
 from .linear import linear
 
@@ -347,7 +347,9 @@ class PreNormResidual:
 
     A layer may have no feed-forward (then it has no `ffn_norm` either), and it may end with a
     `token_input`: a part that adds something made from the step's tokens and the finished stream
-    (`forward(x, pending, ctx) -> pending`: it folds the layer's last output into x itself)."""
+    (`forward(x, pending, ctx) -> pending`: it folds the layer's last output into x itself).  Such a part may
+    apply the norm that the next layer begins with (`ctx.next_input_norm`) at the end of its own last kernel and
+    leave the activations on the step's context; a layer that finds them there, made with its norm, starts from them."""
 
     PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "mixer_norm": "norm", "ffn_norm": "norm",
                   "token_input": "token_input"}
@@ -370,9 +372,17 @@ class PreNormResidual:
             out["token_input"] = self.token_input
         return out
 
+    def input_norm(self) -> Part:
+        """The norm this layer begins with: the layer before may apply it at the end of its own last kernel."""
+        return self.mixer_norm
+
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
                 writes_cache: bool = True) -> Optional[torch.Tensor]:
-        h = self.mixer_norm.forward(x, pending)
+        ready = ctx.shared.pop(NORMED_STREAM, None) if getattr(ctx, "shared", None) else None
+        if ready is not None and ready[1] is self.mixer_norm and pending is None:
+            h = ready[0]                            # the layer before has made it, with this layer's norm
+        else:
+            h = self.mixer_norm.forward(x, pending)
         a = self.mixer.forward(h, ctx, cache, writes_cache)
         if self.ffn is not None:
             h = self.ffn_norm.forward(x, a)

@@ -18,7 +18,7 @@ import torch
 
 from .. import ops
 from ..registry import register_part
-from .base import ParamRequest, Part, Runtime, StepCost
+from .base import NORMED_STREAM, ParamRequest, Part, Runtime, StepCost
 from .linear import linear
 
 
@@ -57,7 +57,14 @@ class GatedSideEmbedding(Part):
         g = ops.gelu_mul_rows(z, self.table, self.offset, ctx.token_ids, self.rt.empty(tuple(z.shape)), ctx.src_row,
                               ctx.prev_tokens)
         y = linear(g, self.w_proj, partial_ok=True)
-        ops.output_norm_add(x, y, self.norm_w, self.ones, self.eps, None)
+        following = getattr(ctx, "next_input_norm", None)
+        if getattr(following, "weight_f32", None) is not None and following.size == self.hidden_size:
+            # the norm that the next layer begins with, in the same kernel
+            h = ops.output_norm_add(x, y, self.norm_w, self.ones, self.eps, self.rt.empty(tuple(x.shape)),
+                                    following.weight_f32, following.eps)
+            ctx.shared[NORMED_STREAM] = (h, following)
+        else:
+            ops.output_norm_add(x, y, self.norm_w, self.ones, self.eps, None)
         return None
 
 
