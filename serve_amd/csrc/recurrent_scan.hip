@@ -210,7 +210,7 @@ static void launch_scan_r(int rpt, int cpt, const void* q, const void* k, const 
 // itself.  A pass that the segment's end cuts short is filled with tokens that change nothing (q = k = v = 0,
 // decay 1).
 //
-// grid (ceil(dv / 64), H, B), 256 threads: wave w owns 16 columns and keeps their S in the registers of the matrix
+// grid (ceil(dv / 64), H, B x pieces), 256 threads: wave w owns 16 columns and keeps their S in the registers of the matrix
 // cores' result layout (lane (g, j): rows 16 m + 4 g + r, column j), which serves as the second operand of
 // S0^T q directly when the contraction runs over the rows in that same order.  All waves share the scaled q and k
 // of the pass in LDS; the next pass's inputs are loaded into registers while this one's products run.  A request's
