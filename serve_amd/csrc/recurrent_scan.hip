@@ -592,7 +592,36 @@ __global__ __launch_bounds__(256) void ssm_prepare_kernel(
     __syncthreads();
   }
   if (c >= C + H) return;
-  for (int t = blockIdx.x * per; t < t_end; ++t) {
+  // A run of tokens inside one segment, none of them among its first taps - 1: every input comes from the step's own
+  // rows.  The channel's inputs of the run and its taps are loaded once, all at a go, and each token is a window of them.
+  const int t_first = blockIdx.x * per;
+  if (per == RS_PREP_TOKENS && t_end - t_first == RS_PREP_TOKENS && c < C) {
+    const int seg = seg_of_token[t_first];
+    if (seg_of_token[t_end - 1] == seg && t_first - (taps - 1) >= cu_q[seg]) {
+      float xin[RS_PREP_TOKENS + RS_MAX_TAPS - 1], w[RS_MAX_TAPS];
+      const TA* src = zx + (size_t)(t_first - (taps - 1)) * zs + col0 + c;
+#pragma unroll
+      for (int i = 0; i < RS_PREP_TOKENS + RS_MAX_TAPS - 1; ++i)
+        if (i < RS_PREP_TOKENS + taps - 1) xin[i] = to_float(src[(size_t)i * zs]);
+#pragma unroll
+      for (int j = 0; j < RS_MAX_TAPS; ++j)
+        if (j < taps) w[j] = conv_w[(size_t)c * taps + j];
+      const float bias = conv_b ? conv_b[c] : 0.f;
+#pragma unroll
+      for (int tt = 0; tt < RS_PREP_TOKENS; ++tt) {
+        float acc = bias;
+#pragma unroll
+        for (int j = 0; j < RS_MAX_TAPS; ++j)
+          if (j < taps) acc = fmaf(w[j], xin[tt + j], acc);
+        const float y = rs_silu(acc);
+        const int t = t_first + tt;
+        xbc[(size_t)t * C + c] = y;
+        if (c < H * P) vout[(size_t)t * H * P + c] = sdt[tt][c / P - h_first] * y;
+      }
+      return;
+    }
+  }
+  for (int t = t_first; t < t_end; ++t) {
     if (c >= C) {
       const int h = c - C;
       const float dt = rs_softplus(dtraw[(size_t)t * H + h] + dt_bias[h]);

@@ -434,15 +434,17 @@ def test_stream_kernels(dtype, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,P,N,G,taps,norm_groups", [(4, 16, 16, 2, 4, 2), (3, 32, 8, 1, 2, 3), (2, 9, 5, 2, 1, 1)])
-def test_state_space_kernels_in_two_steps(dtype, H, P, N, G, taps, norm_groups):
+@pytest.mark.parametrize("lens", [[[9, 1], [1, 6]], [[290, 1], [3, 270]]], ids=["short", "long"])
+@pytest.mark.parametrize("H,P,N,G,taps,norm_groups", [(4, 16, 16, 2, 4, 2), (3, 32, 8, 1, 2, 3), (2, 9, 5, 2, 1, 1), (5, 64, 16, 1, 16, 1)])
+def test_state_space_kernels_in_two_steps(dtype, H, P, N, G, taps, norm_groups, lens):
     """ssm_prepare, conv_state_update, decay_scan and gated_group_norm over two steps against the plain mixer's
-    inner part over the whole sequences (the convolution's last inputs and the state carry over)."""
+    inner part over the whole sequences (the convolution's last inputs and the state carry over).  `long`: steps of
+    more than 256 tokens, whose preparation takes runs of eight tokens (inside a segment from loaded windows, at a
+    segment's first tokens and where two segments meet one by one)."""
     from serve_amd import ops
     torch.manual_seed(P)
     inner, C = H * P, H * P + 2 * G * N
-    lens = [[9, 1], [1, 6]]
-    total = [10, 7]
+    total = [lens[0][0] + lens[1][0], lens[0][1] + lens[1][1]]
     zx = [torch.randn(n, inner + C).to(dtype).double() for n in total]
     dt = [torch.randn(n, H).float().double() for n in total]
     f64 = lambda *s: torch.randn(*s).float().double()   # noqa: E731
