@@ -259,7 +259,11 @@ __global__ __launch_bounds__(256) void decay_scan_block_kernel(
     return (((size_t)h * seq_tiles + col / (16 * CPT)) * RPT + row % RPT) * (size_t)(256 * CPT) +
            (size_t)(((col / CPT) % 16) * 16 + row / RPT) * CPT + col % CPT;
   };
-  float* const mine = scratch + (size_t)blockIdx.z * scratch_stride;      // this piece's row of the scratch
+  // this piece's row of the scratch: the segments that are cut have `pieces` rows each, in their order
+  int cut_before = 0;
+  if (split)
+    for (int s2 = 0; s2 < seg; ++s2) cut_before += (cu_q[s2 + 1] - cu_q[s2] > piece) ? 1 : 0;
+  float* const mine = scratch + (size_t)(cut_before * pieces + pj) * scratch_stride;
   float* st = col >= dv ? nullptr : (split ? mine : (slot >= 0 ? state + (size_t)slot * state_stride : nullptr));
   rs_f4 S[NT];
 #pragma unroll
@@ -435,6 +439,8 @@ __global__ __launch_bounds__(256) void decay_scan_chain_kernel(float* __restrict
   const int at = blockIdx.x * 256 + threadIdx.x;
   if (whole <= piece || at >= floats) return;
   const int count = (whole + piece - 1) / piece;
+  int cut_before = 0;
+  for (int s2 = 0; s2 < seg; ++s2) cut_before += (cu_q[s2 + 1] - cu_q[s2] > piece) ? 1 : 0;
   // at = ((h tiles + tile) RPT + ii) 256 CPT + thread CPT + cc, thread = 16 (column group) + r: row r RPT + ii
   const int per = 256 * CPT;
   const int hi = at / per, thread = (at - hi * per) / CPT;
@@ -442,7 +448,7 @@ __global__ __launch_bounds__(256) void decay_scan_chain_kernel(float* __restrict
   const int slot = state_slots[seg];
   float S = slot >= 0 ? state[(size_t)slot * state_stride + at] : 0.f;
   for (int pj = 0; pj < count; ++pj) {
-    float* mine = scratch + (size_t)(seg * pieces + pj) * scratch_stride;
+    float* mine = scratch + (size_t)(cut_before * pieces + pj) * scratch_stride;
     const float add = mine[at], D = mine[scratch_decays + (size_t)h * DKP + row];
     mine[at] = S;
     S = fmaf(D, S, add);
@@ -493,7 +499,7 @@ extern "C" int sa_decay_scan(const void* q, const void* k, const void* v, int dt
   if (max_q >= RS_BLOCK_MIN_TOKENS && dk <= RS_BLOCK_MAX_DK && (dtype == SA_F32 || dtype == SA_BF16) &&
       q_stride < far_stride && k_stride < far_stride && v_stride < far_stride && (long long)H * dk < far_stride) {
     // piece > 0: segments longer than `piece` tokens (a multiple of 16) run as pieces side by side; scratch: fp32 rows
-    // of scratch_stride >= state floats + H 16 rpt floats, one per (segment, piece), B ceil(max_q / piece) of them
+    // of scratch_stride >= state floats + H 16 rpt floats, ceil(max_q / piece) for every segment that is cut, zeroed
     const long long floats = sa_decay_scan_state_floats(H, dk, dv);
     int pieces = 1;
     if (piece > 0 && max_q > piece) {

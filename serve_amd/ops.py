@@ -743,7 +743,9 @@ SCAN_MAX_DIM = 256
 SCAN_MAX_TAPS = 16
 SCAN_BLOCK_MIN_TOKENS = 6        # csrc/recurrent_scan.hip: RS_BLOCK_MIN_TOKENS
 SCAN_PIECE_MIN = 64              # the shortest piece that a long segment is cut into
-SCAN_PIECE_GROUPS = 512          # workgroups that a step's recurrence should at least have
+SCAN_PIECE_BUSY = 256            # segments are cut where a step's longest ones have fewer workgroups than this (a CU each) ...
+SCAN_PIECE_GROUPS = 512          # ... into so many pieces that they have this many (with 256 and more, cutting lost: 288 -> 389 us)
+SCAN_PIECE_SCRATCH_BYTES = 1 << 30
 
 
 def _pow2_rows(dk: int) -> int:
@@ -806,14 +808,16 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
     # pieces that run side by side (each piece's own contribution to the state first, a chain through them, then the
     # pieces again from their true states), through a scratch row per piece
     piece, scratch = 0, None
-    groups = B * heads * -(-dv // 64)
-    if max_q >= 2 * SCAN_PIECE_MIN and groups < SCAN_PIECE_GROUPS and dk <= 128 and piece_ok:
-        want = -(-SCAN_PIECE_GROUPS // groups)
+    q_lens = list(getattr(ctx, "q_lens", None) or [max_q] * B)       # (bounds, where the step is replayed from a graph)
+    busy = sum(1 for n in q_lens if 2 * n >= max_q) * heads * -(-dv // 64)     # what the longest segments have to run on
+    if max_q >= 2 * SCAN_PIECE_MIN and busy < SCAN_PIECE_BUSY and dk <= 128 and piece_ok:
+        want = -(-SCAN_PIECE_GROUPS // busy)
         piece = max(SCAN_PIECE_MIN, -(-(-(-max_q // want)) // 16) * 16)
-        if max_q > piece:
-            rows = B * -(-max_q // piece)
-            scratch = torch.zeros((rows, need + heads * 16 * _pow2_rows(dk)),
-                                  dtype=torch.float32, device=out.device)
+        cut = sum(1 for n in q_lens if n > piece)
+        rows = cut * -(-max_q // piece)
+        row = need + heads * 16 * _pow2_rows(dk)
+        if max_q > piece and cut > 0 and rows * row * 4 <= SCAN_PIECE_SCRATCH_BYTES:
+            scratch = torch.zeros((rows, row), dtype=torch.float32, device=out.device)
         else:
             piece = 0
     _ret(lib.sa_decay_scan(_ptr(q), _ptr(k), _ptr(v), c_int(_code(q)), LL(q.stride(0)), LL(k.stride(0)), LL(v.stride(0)),

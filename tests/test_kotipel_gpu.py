@@ -274,7 +274,7 @@ def _ctx(lens, slots):
         cu.append(cu[-1] + n)
     seg = [i for i, n in enumerate(lens) for _ in range(n)]
     dev = dict(dtype=torch.int32, device="cuda")
-    return SimpleNamespace(num_tokens=T, num_segments=len(lens), max_q_len=max(lens),
+    return SimpleNamespace(num_tokens=T, num_segments=len(lens), max_q_len=max(lens), q_lens=list(lens),
                            seg_of_token=torch.tensor(seg, **dev), cu_q=torch.tensor(cu, **dev),
                            state_slots=torch.tensor(slots, **dev))
 
