@@ -51,6 +51,8 @@ class RunEntry:
     # row of the model's table of pass vectors (`ModelSpec.pass_vectors`) that is added to the residual stream
     # right before this entry runs (a group of layers that runs several times marks each pass this way)
     pass_vector: Optional[int] = None
+    # with a pass vector: the embedding's output (the stream as it was before the first layer) is added as well
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

@@ -30,7 +30,7 @@ template <typename TA>
 __global__ __launch_bounds__(256) void latent_kv_write_kernel(
     const TA* __restrict__ z, const float* __restrict__ w, const int* __restrict__ positions,
     const float* __restrict__ inv_freq, const int* __restrict__ slot, TA* __restrict__ k_pages,
-    TA* __restrict__ v_pages, float eps, int R, int dr, int Dp, int page_size) {
+    TA* __restrict__ v_pages, float eps, int R, int dr, int Dp, int page_size, float magnitude) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const int s = slot[t];
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(
       float sn, cs;
       sincos_for<TA>(pos * inv_freq[jf], &sn, &cs);
       const float a = to_float(zr[R + jf]), b = to_float(zr[R + jf + half]);
-      kvv = jr < half ? a * cs - b * sn : b * cs + a * sn;
+      kvv = (jr < half ? a * cs - b * sn : b * cs + a * sn) * magnitude;
     }
     kp[i] = from_float<TA>(kvv);
     vp[(size_t)i * page_size] = from_float<TA>(vvv);
@@ -67,16 +67,16 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(
 
 extern "C" int sa_latent_kv_write(const void* z, int act_dtype, const float* w, const int* positions,
                                   const float* inv_freq, const int* slot, void* k_pages, void* v_pages, float eps,
-                                  int T, int R, int dr, int Dp, int page_size, hipStream_t stream) {
+                                  int T, int R, int dr, int Dp, int page_size, float magnitude, hipStream_t stream) {
   if (T <= 0) return 0;
   if (R <= 0 || dr < 0 || (dr & 1) || Dp < R + dr || page_size <= 0) return SA_ERR_ARG;
   dim3 grid(T), block(Dp > 128 ? 256 : 64);
   if (act_dtype == SA_F32)
     hipLaunchKernelGGL(latent_kv_write_kernel<float>, grid, block, 0, stream, (const float*)z, w, positions, inv_freq,
-                       slot, (float*)k_pages, (float*)v_pages, eps, R, dr, Dp, page_size);
+                       slot, (float*)k_pages, (float*)v_pages, eps, R, dr, Dp, page_size, magnitude);
   else if (act_dtype == SA_BF16)
     hipLaunchKernelGGL(latent_kv_write_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)z, w, positions,
-                       inv_freq, slot, (bf16_t*)k_pages, (bf16_t*)v_pages, eps, R, dr, Dp, page_size);
+                       inv_freq, slot, (bf16_t*)k_pages, (bf16_t*)v_pages, eps, R, dr, Dp, page_size, magnitude);
   else return SA_ERR_UNSUPPORTED;
   SA_LAUNCH_CHECK();
   return 0;
@@ -96,6 +96,7 @@ struct HeadTail {
   const int* positions;      // nullptr: no tail
   const float* inv_freq;     // [rot / 2]
   int rot, tail;
+  float magnitude;           // multiplies sine and cosine
 };
 
 template <typename TA>
@@ -110,7 +111,7 @@ __device__ __forceinline__ void write_tail(const HeadTail& ht, const TA* __restr
       float sn, cs;
       sincos_for<TA>(pos * ht.inv_freq[jf], &sn, &cs);
       const float a = to_float(src[jf]), b = to_float(src[jf + half]);
-      v = i < half ? a * cs - b * sn : b * cs + a * sn;
+      v = (i < half ? a * cs - b * sn : b * cs + a * sn) * ht.magnitude;
     }
     dst[i] = from_float<TA>(v);
   }
@@ -197,11 +198,11 @@ __global__ __launch_bounds__(256) void head_linear_small_kernel(const TA* __rest
 
 extern "C" int sa_head_linear(const void* in, int is, int ihs, const void* W, void* out, int os, int ohs,
                               int act_dtype, int T, int H, int K, int N, const int* positions, const float* inv_freq,
-                              int rot, int tail, hipStream_t stream) {
+                              int rot, int tail, float magnitude, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || K <= 0 || N <= 0 || H > 65535 || (N + 255) / 256 > 65535) return SA_ERR_ARG;
   if (positions && ((!inv_freq && rot > 0) || rot < 0 || (rot & 1) || tail < rot)) return SA_ERR_ARG;
-  HeadTail ht = {positions, inv_freq, rot, tail};
+  HeadTail ht = {positions, inv_freq, rot, tail, magnitude};
   if (T <= 64 && K <= HL_SMALL_K) {
     dim3 grid(T, H), block(256);
     if (act_dtype == SA_F32)

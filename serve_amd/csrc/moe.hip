@@ -1,7 +1,9 @@
 // Routed experts: every token takes the `top` experts with the largest router logits, weighted by the
 // softmax over those logits alone (or: by their shares of the softmax over all experts, divided by the sum
-// of the chosen shares + 1e-20; either way times a constant); an expert is down(gate(gate x, up x)) with
-// one of the gates of common.h (silu(g) u and others).
+// of the chosen shares + 1e-20; or: by the sigmoid of each chosen logit as it is; each times a constant); an expert
+// is down(gate(gate x, up x)) with one of the gates of common.h (silu(g) u and others).  The weight multiplies the
+// expert's output (in `combine`), or, where a design says so, its input: gate and up are linear in x, so
+// expert(w x) = down(gate(w gate x, w up x)), and the weight enters where the gate is applied.
 //
 // Nothing is read back to the host: the tokens are grouped by expert on the device, and the
 // products run over a list of (expert, rows) tiles that is built there, from a grid sized for
@@ -25,10 +27,11 @@
 // ---------------------------------------------------------------------------------------------
 // route: a wave per token.  Ties go to the lower index.
 // ---------------------------------------------------------------------------------------------
-// over_all: the weights are shares of the softmax over all E logits, renormalised over the chosen ones
-// (p_k / S) / (sum_chosen p / S + 1e-20) with S the sum over all; else p_k / sum_chosen p.  Both times wscale.
+// mode 1: the weights are shares of the softmax over all E logits, renormalised over the chosen ones
+// (p_k / S) / (sum_chosen p / S + 1e-20) with S the sum over all; mode 0: p_k / sum_chosen p; mode 2: the sigmoid of
+// every chosen logit, not normalised.  All times wscale.
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
-                                            int E, int top, int lane, int over_all, float wscale);
+                                            int E, int top, int lane, int mode, float wscale);
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldz, int* __restrict__ ids,
                                                         float* __restrict__ wts, int T, int E, int top, int over_all,
@@ -40,7 +43,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 }
 
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __restrict__ ids, float* __restrict__ wts,
-                                            int E, int top, int lane, int over_all, float wscale) {
+                                            int E, int top, int lane, int mode, float wscale) {
+  const int over_all = mode == 1;
   float prev_v = INFINITY;
   int prev_i = -1;
   float first = 0.f, sum = 0.f;
@@ -60,7 +64,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __
       if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
     if (k == 0) first = bv;
-    const float p = expf(bv - first);
+    const float p = mode == 2 ? 1.f / (1.f + expf(-bv)) : expf(bv - first);
     sum += p;
     if (lane == 0) {
       ids[k] = bi;
@@ -76,7 +80,9 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int* __
     for (int e = lane; e < E; e += SA_WAVE) part += expf(z[e] - first);
     all = wave_sum(part);
   }
-  if (lane == 0) {
+  if (lane == 0 && mode == 2) {
+    for (int k = 0; k < top; ++k) wts[k] *= wscale;
+  } else if (lane == 0) {
     const float denom = over_all ? sum / all + 1e-20f : sum;
     for (int k = 0; k < top; ++k) wts[k] = ((over_all ? wts[k] / all : wts[k]) / denom) * wscale;
   }
@@ -192,7 +198,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TA* __restrict__
                                                           const int* __restrict__ perm, const int* __restrict__ tile_expert,
                                                           const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
                                                           TA* __restrict__ act, int top, int d, int F, int gate_kind,
-                                                          float gate_limit) {
+                                                          float gate_limit, const float* __restrict__ in_wts) {
   __shared__ float sa[MOE_TK][MOE_TM + 1];
   __shared__ float sw0[MOE_TK][MOE_TN + 1];
   __shared__ float sw1[MOE_TK][MOE_TN + 1];
@@ -211,11 +217,12 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const TA* __restrict__
   for (int rr = 0; rr < 2; ++rr) {
     const int r = ty + 16 * rr;
     if (r >= rows) continue;
+    const float w = in_wts ? in_wts[perm[row0 + r]] : 1.f;          // (the weight on the expert's input)
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int n = n0 + tx + 16 * c;
       if (n < F) {
-        act[(size_t)(row0 + r) * F + n] = from_float<TA>(gate_mul(g[rr][c], u[rr][c], gate_kind, gate_limit));
+        act[(size_t)(row0 + r) * F + n] = from_float<TA>(gate_mul(g[rr][c] * w, u[rr][c] * w, gate_kind, gate_limit));
       }
     }
   }
@@ -280,7 +287,8 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
                                                        const int* __restrict__ perm, const int* __restrict__ tile_expert,
                                                        const int* __restrict__ tile_row0, const int* __restrict__ num_tiles,
                                                        bf16_t* __restrict__ act, float* __restrict__ yk, int top, int N,
-                                                       int K, int gate_kind, float gate_limit) {
+                                                       int K, int gate_kind, float gate_limit,
+                                                       const float* __restrict__ in_wts) {
   // WR: groups of 16 weight rows a wave owns (per matrix); KU: steps of 32 along K whose loads are in flight together
   constexpr int NM = GATE_UP ? 2 : 1;
   constexpr int RT = NM * WR;
@@ -368,6 +376,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + c;
     if (m >= rows) continue;
+    const float w = GATE_UP && in_wts ? in_wts[perm[row0 + m]] : 1.f;          // (the weight on the expert's input)
 #pragma unroll
     for (int wr = 0; wr < WR; ++wr) {
       const int n = n0 + wr * 16 + 4 * g;
@@ -376,7 +385,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           if (n + r < N)
-            dst[r] = from_float<bf16_t>(gate_mul(acc[wr][mt][r], acc[RT - WR + wr][mt][r], gate_kind, gate_limit));
+            dst[r] = from_float<bf16_t>(gate_mul(acc[wr][mt][r] * w, acc[RT - WR + wr][mt][r] * w, gate_kind, gate_limit));
       } else {
         float* dst = yk + (size_t)perm[row0 + m] * N + n;
 #pragma unroll
@@ -387,7 +396,8 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
   }
 }
 
-// combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate).
+// combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate);
+// wts null: the rows are added as they are (their weights went into the experts' inputs).
 // TOPMAX / PMAX: upper bounds of `top` / `parts` (0: any number, in a loop): with bounds, all loads of an output
 // are issued before anything is added (rows beyond the bounds are read from a clamped place and dropped).
 template <typename TS, int TOPMAX, int PMAX>
@@ -401,7 +411,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   if (TOPMAX > 0) {
     float wk[TOPMAX > 0 ? TOPMAX : 1];
 #pragma unroll
-    for (int k = 0; k < TOPMAX; ++k) wk[k] = k < top ? wts[(size_t)t * top + k] : 0.f;
+    for (int k = 0; k < TOPMAX; ++k) wk[k] = k < top ? (wts ? wts[(size_t)t * top + k] : 1.f) : 0.f;
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
       float a[TOPMAX > 0 ? TOPMAX : 1], sp[PMAX];
 #pragma unroll
@@ -420,7 +430,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   }
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float v = 0.f;
-    for (int k = 0; k < top; ++k) v += wts[(size_t)t * top + k] * yk[((size_t)t * top + k) * d + i];
+    for (int k = 0; k < top; ++k) v += (wts ? wts[(size_t)t * top + k] : 1.f) * yk[((size_t)t * top + k) * d + i];
     if (shared) {
       float sh = 0.f;
       for (int p = 0; p < parts; ++p) sh += to_float(shared[p * part_stride + (size_t)t * d + i]);
@@ -449,6 +459,7 @@ extern "C" int sa_moe_route(const float* logits, int ldz, int* ids, float* wts, 
 #define MOE_SMALL_ROWS 1024
 
 // logits != nullptr (and T <= MOE_ROUTE_INSIDE): ids and wts are made here from the router's logits fp32 [T, ldz]
+// (over_all: the mode of route_token, 0 to 2).  in_wts (fp32 [T top], may be wts itself): the weights multiply the experts' inputs
 #define MOE_ROUTE_INSIDE 16
 
 extern "C" int sa_moe_route_inside_limit() { return MOE_ROUTE_INSIDE; }
@@ -456,7 +467,7 @@ extern "C" int sa_moe_route_inside_limit() { return MOE_ROUTE_INSIDE; }
 extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void* Wg, const void* Wu,
                               const void* Wd, int* ints, void* act, float* yk, int T, int top, int E, int d, int F,
                               const float* logits, int ldz, float* wts, int over_all, float wscale, int gate_kind,
-                              float gate_limit, hipStream_t stream) {
+                              float gate_limit, const float* in_wts, hipStream_t stream) {
   if (T <= 0) return 0;
   const long long n = (long long)T * top;
   if (E <= 0 || top <= 0 || d <= 0 || F <= 0 || n > 0x3fffffffLL) return SA_ERR_ARG;
@@ -488,10 +499,11 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   do {                                                                                                                 \
     hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, true, WR, KU>), g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,     \
                        (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, nullptr,     \
-                       top, F, d, gate_kind, gate_limit);                                                              \
+                       top, F, d, gate_kind, gate_limit, in_wts);                                                      \
     SA_LAUNCH_CHECK();                                                                                                 \
     hipLaunchKernelGGL((moe_mfma_kernel<MT, KS, false, WR, KU>), g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd,  \
-                       nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F, 0, 0.f);     \
+                       nullptr, offsets, perm, tile_expert, tile_row0, num_tiles, nullptr, yk, top, d, F, 0, 0.f,      \
+                       nullptr);                                                                                       \
   } while (0)
     if (small) GO(1, 4, 1, 2);
     else GO(4, 1, 4, 2);
@@ -504,14 +516,14 @@ extern "C" int sa_moe_experts(const void* h, int act_dtype, int* ids, const void
   if (act_dtype == SA_F32) {
     hipLaunchKernelGGL(moe_gate_up_kernel<float>, g1, block, 0, stream, (const float*)h, (const float*)Wg,
                        (const float*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (float*)act, top, d, F,
-                       gate_kind, gate_limit);
+                       gate_kind, gate_limit, in_wts);
     SA_LAUNCH_CHECK();
     hipLaunchKernelGGL(moe_down_kernel<float>, g2, block, 0, stream, (const float*)act, (const float*)Wd, offsets, perm,
                        tile_expert, tile_row0, num_tiles, yk, d, F);
   } else if (act_dtype == SA_BF16) {
     hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, g1, block, 0, stream, (const bf16_t*)h, (const bf16_t*)Wg,
                        (const bf16_t*)Wu, offsets, perm, tile_expert, tile_row0, num_tiles, (bf16_t*)act, top, d, F,
-                       gate_kind, gate_limit);
+                       gate_kind, gate_limit, in_wts);
     SA_LAUNCH_CHECK();
     hipLaunchKernelGGL(moe_down_kernel<bf16_t>, g2, block, 0, stream, (const bf16_t*)act, (const bf16_t*)Wd, offsets,
                        perm, tile_expert, tile_row0, num_tiles, yk, d, F);

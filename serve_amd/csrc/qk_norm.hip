@@ -389,3 +389,113 @@ extern "C" int sa_head_gate(void* a, const void* g, int dtype, long long g_strid
   SA_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Biases, a rotation of part of every head with a magnitude, and the cache write with padding, for an attention
+// without norms on its queries and keys.  Rows qkv [T, Hq D | Hk D | Hk Dv] (row_stride elements apart):
+//   value = qkv + bias (bias fp32 over the whole row, may be null)
+//   the first `rot` dims of every query and key head turn by position * freq[j]; pair j is (j, j + rot / 2), or
+//   (2j, 2j + 1) with `adjacent`; sine and cosine are multiplied by `magnitude`
+// Queries go to q_out [T, Hq Dp], keys to k_pages [P, Hk, page, Dp], values to v_pages [P, Hk, Dp, page], each head
+// padded with zeros up to Dp.  slot null: queries only; slot[t] < 0: nothing of token t is stored.
+// Queries and keys: a thread an element of the padded output, the first element of a pair computes and writes both.
+// Values: the last blocks of the grid, neighbouring lanes on neighbouring tokens (the tokens of a page lie side by
+// side in the transposed value pages).
+// ---------------------------------------------------------------------------------------------
+template <typename TA, bool EXACT>
+__global__ __launch_bounds__(256) void bias_rope_kv_write_kernel(
+    const TA* __restrict__ qkv, long long row_stride, TA* __restrict__ q_out, const int* __restrict__ positions,
+    const int* __restrict__ slot, TA* __restrict__ k_pages, TA* __restrict__ v_pages, const float* __restrict__ bias,
+    const float* __restrict__ freq, int rot, int adjacent, float magnitude, int T, int Hq, int Hk, int D, int Dv, int Dp,
+    int page_size, long long qk_blocks) {
+  const TA zero = from_float<TA>(0.f);
+  const int units = Hq + (slot ? Hk : 0);
+  if ((long long)blockIdx.x < qk_blocks) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)T * units * Dp) return;
+    const int i = (int)(idx % Dp);
+    const long long tu = idx / Dp;
+    const int u = (int)(tu % units), t = (int)(tu / units);
+    const bool is_q = u < Hq;
+    const int g = is_q ? u : u - Hq;
+    TA* dst;
+    if (is_q) {
+      dst = q_out + ((size_t)t * Hq + g) * Dp;
+    } else {
+      const int s = slot[t];
+      if (s < 0) return;
+      const int page = s / page_size, off = s - page * page_size;
+      dst = k_pages + (((size_t)page * Hk + g) * page_size + off) * Dp;
+    }
+    if (i >= D) {
+      dst[i] = zero;
+      return;
+    }
+    const size_t col = (is_q ? 0 : (size_t)Hq * D) + (size_t)g * D;
+    const TA* x = qkv + (size_t)t * row_stride + col;
+    const float* b = bias ? bias + col : nullptr;
+    if (i >= rot) {
+      dst[i] = from_float<TA>(to_float(x[i]) + (b ? b[i] : 0.f));
+      return;
+    }
+    const int half = rot >> 1;
+    const bool first = adjacent ? (i & 1) == 0 : i < half;
+    if (!first) return;                              // (its partner writes both)
+    const int ip = adjacent ? i + 1 : i + half;
+    const int j = adjacent ? i >> 1 : i;
+    const float a = (float)positions[t] * freq[j];
+    float sn, cs;
+    if (EXACT) sincosf(a, &sn, &cs);
+    else sincos_reduced(a, &sn, &cs);
+    sn *= magnitude;
+    cs *= magnitude;
+    const float p0 = to_float(x[i]) + (b ? b[i] : 0.f), p1 = to_float(x[ip]) + (b ? b[ip] : 0.f);
+    dst[i] = from_float<TA>(p0 * cs - p1 * sn);
+    dst[ip] = from_float<TA>(p1 * cs + p0 * sn);
+    return;
+  }
+  if (!slot) return;
+  const long long idx = ((long long)blockIdx.x - qk_blocks) * blockDim.x + threadIdx.x;
+  if (idx >= (long long)T * Hk * Dp) return;
+  const int t = (int)(idx % T);
+  const int gi = (int)(idx / T);
+  const int g = gi / Dp, i = gi - g * Dp;
+  const int s = slot[t];
+  if (s < 0) return;
+  const int page = s / page_size, off = s - page * page_size;
+  TA out = zero;
+  if (i < Dv) {
+    const size_t col = (size_t)(Hq + Hk) * D + (size_t)g * Dv + i;
+    out = from_float<TA>(to_float(qkv[(size_t)t * row_stride + col]) + (bias ? bias[col] : 0.f));
+  }
+  v_pages[(((size_t)page * Hk + g) * Dp + i) * page_size + off] = out;
+}
+
+extern "C" int sa_bias_rope_kv_write(const void* qkv, long long row_stride, void* q_out, int act_dtype,
+                                     const int* positions, const int* slot, void* k_pages, void* v_pages,
+                                     const float* bias, const float* freq, int rot, int adjacent, float magnitude, int T,
+                                     int Hq, int Hk, int D, int Dv, int Dp, int page_size, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (Hq <= 0 || Hk <= 0 || D <= 0 || Dv <= 0 || Dp < D || Dp < Dv || page_size <= 0 || !q_out || !positions || !qkv)
+    return SA_ERR_ARG;
+  if (row_stride < (long long)Hq * D + (long long)Hk * (D + Dv) || (slot && (!k_pages || !v_pages)) || rot < 0 || rot % 2 ||
+      rot > D || (rot > 0 && !freq))
+    return SA_ERR_ARG;
+  const int threads = 256;
+  const long long qk_blocks = ((long long)T * (Hq + (slot ? Hk : 0)) * Dp + threads - 1) / threads;
+  const long long v_blocks = slot ? ((long long)T * Hk * Dp + threads - 1) / threads : 0;
+  if (qk_blocks + v_blocks > 0x7fffffffLL) return SA_ERR_ARG;
+  dim3 grid((unsigned)(qk_blocks + v_blocks)), block(threads);
+  if (act_dtype == SA_F32)
+    hipLaunchKernelGGL((bias_rope_kv_write_kernel<float, true>), grid, block, 0, stream, (const float*)qkv, row_stride,
+                       (float*)q_out, positions, slot, (float*)k_pages, (float*)v_pages, bias, freq, rot, adjacent,
+                       magnitude, T, Hq, Hk, D, Dv, Dp, page_size, qk_blocks);
+  else if (act_dtype == SA_BF16)
+    hipLaunchKernelGGL((bias_rope_kv_write_kernel<bf16_t, false>), grid, block, 0, stream, (const bf16_t*)qkv,
+                       row_stride, (bf16_t*)q_out, positions, slot, (bf16_t*)k_pages, (bf16_t*)v_pages, bias, freq, rot,
+                       adjacent, magnitude, T, Hq, Hk, D, Dv, Dp, page_size, qk_blocks);
+  else
+    return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

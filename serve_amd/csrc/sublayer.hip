@@ -234,12 +234,19 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
   return 0.5f * z * (1.f + tanhf(u));
 }
 
+// kind 0: gelu (tanh form), 1: silu, 2: the square of relu
+__device__ __forceinline__ float activate(float z, int kind) {
+  if (kind == 0) return gelu_tanh_f(z);
+  if (kind == 1) return z / (1.f + expf(-z));
+  const float r = fmaxf(z, 0.f);
+  return r * r;
+}
+
 template <typename TA>
 __global__ void activation_kernel(TA* __restrict__ a, size_t n, int kind) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     const float z = to_float(a[i]);
-    const float r = kind == 0 ? gelu_tanh_f(z) : z / (1.f + expf(-z));
-    a[i] = from_float<TA>(r);
+    a[i] = from_float<TA>(activate(z, kind));
   }
 }
 
@@ -251,8 +258,7 @@ __global__ __launch_bounds__(256) void activation_bf16x8_kernel(bf16_t* __restri
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const float z0 = bf16_bits_to_float(w[k] & 0xffffu), z1 = bf16_bits_to_float(w[k] >> 16);
-      const float r0 = kind == 0 ? gelu_tanh_f(z0) : z0 / (1.f + expf(-z0));
-      const float r1 = kind == 0 ? gelu_tanh_f(z1) : z1 / (1.f + expf(-z1));
+      const float r0 = activate(z0, kind), r1 = activate(z1, kind);
       w[k] = (uint32_t)float_to_bf16_bits(r0) | ((uint32_t)float_to_bf16_bits(r1) << 16);
     }
     *reinterpret_cast<uint4*>(a + gi * 8) = make_uint4(w[0], w[1], w[2], w[3]);
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(256) void activation_bf16x8_kernel(bf16_t* __restri
 
 extern "C" int sa_activation(void* a, int act_dtype, long long n, int kind, hipStream_t stream) {
   if (n <= 0) return 0;
-  if (kind < 0 || kind > 1) return SA_ERR_ARG;
+  if (kind < 0 || kind > 2) return SA_ERR_ARG;
   if (act_dtype == SA_BF16 && (n & 7) == 0 && ((uintptr_t)a & 15) == 0) {
     long long vb = (n / 8 + 255) / 256;
     if (vb > 65536) vb = 65536;

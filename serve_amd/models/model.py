@@ -53,6 +53,8 @@ class Model:
                 raise ValueError(f"run order names layer {e.layer}, the model has {len(self.layers)}")
             if e.pass_vector is not None and self.pass_vectors is None:
                 raise ValueError("the run order names a pass vector, the model has no table of them")
+            if e.adds_embedding and e.pass_vector is None:
+                raise ValueError("the embedding's output is added again together with a pass vector")
         self._check_cache_owners()
         self.rt: Optional[Runtime] = None
 
@@ -104,15 +106,24 @@ class Model:
     def _cache_owner(self, layer: int) -> Optional[Part]:
         return self.layers[layer].cache_owner()
 
+    def _embedding_state(self) -> Optional[StateRequest]:
+        """Per-request state of the embedding (a part that looks back at a request's earlier tokens), or None."""
+        return self.embedding.state_request() if hasattr(self.embedding, "state_request") else None
+
     def cache_requests(self) -> List[Optional[TokenCacheRequest]]:
-        """Per cache layer: what the part that writes it keeps per token."""
+        """Per cache layer: what the part that writes it keeps per token.  An embedding with per-request state
+        has one more cache layer, the last, that holds nothing per token."""
         owners = [self._cache_owner(l) for l in self._cache_writer_layer]
-        return [None if o is None else o.cache_request() for o in owners]
+        out = [None if o is None else o.cache_request() for o in owners]
+        return out + [None] if self._embedding_state() is not None else out
 
     def state_requests(self) -> List[Optional[StateRequest]]:
-        """Per cache layer: the fixed-size per-request state its part needs."""
+        """Per cache layer: the fixed-size per-request state its part needs (the embedding's, if it has one, in a
+        last cache layer of its own)."""
         owners = [self._cache_owner(l) for l in self._cache_writer_layer]
-        return [None if o is None else o.state_request() for o in owners]
+        out = [None if o is None else o.state_request() for o in owners]
+        emb = self._embedding_state()
+        return out + [emb] if emb is not None else out
 
     # -- what a step costs (for measurements) ---------------------------------------------------
     def step_cost(self, tokens: int, logit_rows: int = 1, context_before: int = 0):
@@ -171,7 +182,17 @@ class Model:
     # -- running -------------------------------------------------------------------------------
     def forward(self, ctx, caches: List[LayerCache]) -> torch.Tensor:
         """Run the tokens of one step; return fp32 logits [R, V] at ctx.logit_rows."""
-        x = self.embedding.forward(ctx)
+        again = any(e.adds_embedding for e in self.spec.run_order)
+        x0 = None
+        if self._embedding_state() is not None:
+            # (its state lies in the cache layer behind the run order's)
+            x = self.embedding.forward(ctx, caches[self.spec.num_cache_layers()], keep=again)
+            if again:
+                x, x0 = x
+        else:
+            x = self.embedding.forward(ctx)
+            if again:
+                x0 = x.clone()
         ctx.stream_copy = None          # (what a layer may leave for the next: the stream in the activation dtype)
         ctx.shared = {}                 # (and what layers leave for later layers of the step, by name)
         pending = None
@@ -184,7 +205,7 @@ class Model:
             if nxt is not None and order[i + 1].pass_vector is not None:
                 ctx.next_input_norm = None          # (the stream changes between the two layers)
             if e.pass_vector is not None:
-                pending = self.pass_vectors.forward(x, pending, e.pass_vector)
+                pending = self.pass_vectors.forward(x, pending, e.pass_vector, x0 if e.adds_embedding else None)
             pending = self.layers[e.layer].forward(x, pending, ctx, caches[e.cache], e.writes_cache)
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)

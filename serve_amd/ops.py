@@ -445,11 +445,12 @@ def output_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], weight: Optional
     return h
 
 
-ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "relu_squared": 2}
 
 
 def activation(a: torch.Tensor, kind: str) -> torch.Tensor:
-    """a = act(a) in place: 'gelu_tanh' (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or 'silu'."""
+    """a = act(a) in place: 'gelu_tanh' (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))), 'silu' or
+    'relu_squared' (max(z, 0)^2)."""
     _dev(a)
     _check(kind in ACTIVATIONS, f"unknown activation {kind!r}; known: {sorted(ACTIVATIONS)}")
     lib = load_library("sublayer")
@@ -511,9 +512,10 @@ def delta_rule(z: torch.Tensor, conv_w: torch.Tensor, ba: torch.Tensor, A_log: t
 
 def latent_kv_write(z: torch.Tensor, norm_w: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
                     slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, eps: float, rank: int,
-                    rot_dim: int) -> None:
+                    rot_dim: int, magnitude: float = 1.0) -> None:
     """z [T, rank + rot_dim] -> the token's cache rows: k_pages [P, 1, page, Dp] gets
-    [normed latent | rotated key part | 0], v_pages [P, 1, Dp, page] the normed latent (and zeros)."""
+    [normed latent | rotated key part | 0], v_pages [P, 1, Dp, page] the normed latent (and zeros).
+    `magnitude` multiplies the rotation's sine and cosine."""
     _dev(z, norm_w, positions, inv_freq, slots, k_pages, v_pages)
     T = z.shape[0]
     _check(z.dim() == 2 and z.shape[1] == rank + rot_dim, f"z must be [T, {rank + rot_dim}]")
@@ -528,17 +530,18 @@ def latent_kv_write(z: torch.Tensor, norm_w: torch.Tensor, positions: torch.Tens
     lib = load_library("latent")
     _ret(lib.sa_latent_kv_write(_ptr(z), c_int(_code(z)), _ptr(norm_w), _ptr(positions), _ptr(inv_freq), _ptr(slots),
                                 _ptr(k_pages), _ptr(v_pages), c_float(eps), c_int(T), c_int(rank), c_int(rot_dim),
-                                c_int(Dp), c_int(page_size), _stream()), "latent_kv_write")
+                                c_int(Dp), c_int(page_size), c_float(magnitude), _stream()), "latent_kv_write")
 
 
 def head_linear(x: torch.Tensor, in_stride: int, in_head_stride: int, w: torch.Tensor, out: torch.Tensor,
                 out_stride: int, out_head_stride: int, T: int, positions: Optional[torch.Tensor] = None,
-                inv_freq: Optional[torch.Tensor] = None, rot: int = 0, tail: int = 0) -> torch.Tensor:
+                inv_freq: Optional[torch.Tensor] = None, rot: int = 0, tail: int = 0,
+                magnitude: float = 1.0) -> torch.Tensor:
     """out[t, h, :N] = x[t, h, :K] @ w[h] for w [H, K, N]: head h's K inputs of token t start at element
     t * in_stride + h * in_head_stride of x, its N outputs at t * out_stride + h * out_head_stride of out.
     With `positions`: behind the N outputs come the `rot` inputs that lie behind the head's K inputs, rotated by
-    the token's position (dimension i with i + rot / 2, angles positions[t] * inv_freq[i]), then zeros up to
-    `tail` places in all."""
+    the token's position (dimension i with i + rot / 2, angles positions[t] * inv_freq[i], sine and cosine times
+    `magnitude`), then zeros up to `tail` places in all."""
     _dev(x, w, out, positions, inv_freq)
     _check(w.dim() == 3 and x.dtype == w.dtype == out.dtype, "head_linear: w must be [H, K, N], one dtype throughout")
     H, K, N = w.shape
@@ -555,8 +558,8 @@ def head_linear(x: torch.Tensor, in_stride: int, in_head_stride: int, w: torch.T
     lib = load_library("latent")
     _ret(lib.sa_head_linear(_ptr(x), c_int(in_stride), c_int(in_head_stride), _ptr(w), _ptr(out), c_int(out_stride),
                             c_int(out_head_stride), c_int(_code(x)), c_int(T), c_int(H), c_int(K), c_int(N),
-                            _ptr(positions), _ptr(inv_freq), c_int(rot), c_int(tail), _stream()),
-         "head_linear")
+                            _ptr(positions), _ptr(inv_freq), c_int(rot), c_int(tail), c_float(magnitude),
+                            _stream()), "head_linear")
     return out
 
 
@@ -653,6 +656,49 @@ def row_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, positions: to
     return q_out
 
 
+def bias_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                       slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                       v_pages: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+                       inv_freq: Optional[torch.Tensor], rot_dim: int, adjacent_pairs: bool, magnitude: float,
+                       num_heads: int, num_kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """From rows qkv [T, Hq D | Hk D | Hk Dv | ...]: plus `bias` (fp32 over the Hq D + Hk (D + Dv) columns, or None); in
+    every query and key head the first `rot_dim` dims rotated by position * inv_freq[j] (pair j = (j, j + rot_dim / 2), or
+    (2j, 2j + 1) with `adjacent_pairs`), sine and cosine times `magnitude`.  Queries go to q_out [T, Hq Dp], keys and
+    values to the token's slot of k_pages [P, Hk, page, Dp] and v_pages [P, Hk, Dp, page], each head padded with
+    zeros up to Dp.  `slots` None: queries only."""
+    _dev(q_out, positions, slots, k_pages, v_pages, bias, inv_freq)
+    Hq, Hk, D, Dv = num_heads, num_kv_heads, dim, vdim
+    T = qkv.shape[0]
+    cols = Hq * D + Hk * (D + Dv)
+    _check(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= cols,
+           f"qkv must be rows of at least {cols} on the GPU")
+    _check(q_out.dim() == 2 and q_out.shape[0] == T and q_out.shape[1] % Hq == 0 and q_out.dtype == qkv.dtype
+           and q_out.is_contiguous(), "q_out must be contiguous [T, Hq Dp] in the dtype of qkv")
+    Dp = q_out.shape[1] // Hq
+    _check(Dp >= D and Dp >= Dv, f"the padded head size {Dp} is below dim {D} or vdim {Dv}")
+    if bias is not None:
+        _f32vec(bias, cols, "bias")
+    _check(rot_dim >= 0 and rot_dim % 2 == 0 and rot_dim <= D, "rot_dim must be even and within dim")
+    if rot_dim:
+        _f32vec(inv_freq, rot_dim // 2, "inv_freq")
+    _i32(positions, T, "positions")
+    page_size = 1
+    if slots is not None:
+        _i32(slots, T, "slots")
+        P, _, page_size, _ = k_pages.shape
+        _check(k_pages.shape == (P, Hk, page_size, Dp) and v_pages.shape == (P, Hk, Dp, page_size),
+               f"the cache must be k [P, {Hk}, page, {Dp}] and v [P, {Hk}, {Dp}, page]")
+        _check(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "cache dtype must match activations")
+    lib = load_library("qk_norm")
+    _ret(lib.sa_bias_rope_kv_write(_ptr(qkv), ctypes.c_longlong(qkv.stride(0)), _ptr(q_out), c_int(_code(qkv)),
+                                   _ptr(positions), _ptr(slots), _ptr(k_pages if slots is not None else None),
+                                   _ptr(v_pages if slots is not None else None), _ptr(bias),
+                                   _ptr(inv_freq if rot_dim else None), c_int(rot_dim), c_int(1 if adjacent_pairs else 0),
+                                   c_float(magnitude), c_int(T), c_int(Hq), c_int(Hk), c_int(D), c_int(Dv), c_int(Dp),
+                                   c_int(page_size), _stream()), "bias_rope_kv_write")
+    return q_out
+
+
 def head_gate(a: torch.Tensor, rows: torch.Tensor, col: int, num_heads: int) -> torch.Tensor:
     """a[t, h, :] *= sigmoid(rows[t, col + h]) in place: a [T, H Dp], the heads' gate logits in the columns
     col .. col + H - 1 of `rows` (which may be a wider product's output)."""
@@ -681,10 +727,11 @@ def _parts_of(y: torch.Tensor, T: int, d: int, what: str):
 
 
 def stream_add(x: torch.Tensor, y: Optional[torch.Tensor], vec: Optional[torch.Tensor] = None,
-               h: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """x += y + vec on the fp32 residual stream x [T, d], in place (y: [T, d] or fp32 [parts, T, d] partial sums, added
-    in order; vec fp32 [d]; either may be None), and `h` ([T, d], any kernel dtype) receives a copy of the new x."""
-    _dev(x, y, vec, h)
+               h: Optional[torch.Tensor] = None, extra: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += y + vec + extra on the fp32 residual stream x [T, d], in place (y: [T, d] or fp32 [parts, T, d] partial sums,
+    added in order; vec fp32 [d]; extra fp32 [T, d]; each may be None), and `h` ([T, d], any kernel dtype) receives a
+    copy of the new x."""
+    _dev(x, y, vec, h, extra)
     _check(x.dtype == torch.float32 and x.dim() == 2, "residual stream must be fp32 [T, d]")
     T, d = x.shape
     parts, ycode = 1, F32
@@ -694,10 +741,50 @@ def stream_add(x: torch.Tensor, y: Optional[torch.Tensor], vec: Optional[torch.T
         _f32vec(vec, d, "the row vector")
     if h is not None:
         _check(h.shape == (T, d), "the stream's copy must be [T, d]")
+    if extra is not None:
+        _check(extra.dtype == torch.float32 and extra.shape == (T, d) and extra.is_contiguous(),
+               "the second array must be contiguous fp32 [T, d]")
     lib = load_library("stream_ops")
-    _ret(lib.sa_stream_add(_ptr(x), _ptr(y), c_int(ycode), c_int(parts), _ptr(vec), _ptr(h),
+    _ret(lib.sa_stream_add(_ptr(x), _ptr(y), c_int(ycode), c_int(parts), _ptr(vec), _ptr(extra), _ptr(h),
                            c_int(_code(h) if h is not None else F32), c_int(T), c_int(d), _stream()), "stream_add")
     return h
+
+
+def pair_embed(table: torch.Tensor, pair_table: torch.Tensor, ctx, last: torch.Tensor, out: torch.Tensor,
+               mul_prev: int, mul_cur: int, keep: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = table[tok_t] + pair_table[(prev_t * mul_prev + tok_t * mul_cur) mod buckets] as fp32, with
+    pair_table [buckets + 1, d] whose last row serves a sequence's first token (position 0).  prev_t is the token
+    before t in its segment, or what `last` (int32 [slots, 1], by the segment's state slot) holds for the segment's
+    first token; afterwards `last` holds every segment's last token.  `ctx`: the step (token_ids, positions,
+    seg_of_token, cu_q, state_slots, src_row / prev_tokens for tokens sampled on the device).  `keep`: a second
+    copy of the result (fp32 [T, d])."""
+    _dev(table, pair_table, last, out, keep, ctx.token_ids, ctx.positions, ctx.seg_of_token, ctx.cu_q, ctx.state_slots,
+         ctx.src_row, ctx.prev_tokens)
+    T, B = ctx.token_ids.numel(), ctx.state_slots.numel()
+    _check(table.dim() == 2 and pair_table.dim() == 2 and pair_table.shape[1] == table.shape[1]
+           and pair_table.shape[0] >= 2 and table.dtype == pair_table.dtype and table.is_contiguous()
+           and pair_table.is_contiguous(), "the tables must be [V, d] and [buckets + 1, d] of one dtype")
+    V, d = table.shape
+    _check(out.dtype == torch.float32 and out.shape == (T, d) and out.is_contiguous(), "the output must be fp32 [T, d]")
+    if keep is not None:
+        _check(keep.dtype == torch.float32 and keep.shape == (T, d) and keep.is_contiguous(), "the copy must be fp32 [T, d]")
+    _check(last.dtype == torch.int32 and last.is_contiguous() and last.dim() == 2 and last.shape[1] == 1,
+           "the previous tokens must be int32 [slots, 1]")
+    _check(mul_prev >= 0 and mul_cur >= 0, "the multipliers must not be negative")
+    for name in ("token_ids", "positions", "seg_of_token"):
+        _i32(getattr(ctx, name), T, name)
+    _i32(ctx.cu_q, B + 1, "cu_q")
+    _i32(ctx.state_slots, B, "state_slots")
+    if ctx.src_row is not None:
+        _i32(ctx.src_row, T, "src_row")
+        _check(ctx.prev_tokens is not None and ctx.prev_tokens.dtype == torch.int32, "sampled tokens must be int32")
+    lib = load_library("stream_ops")
+    _ret(lib.sa_pair_embed(_ptr(table), _ptr(pair_table), c_int(_code(table)), _ptr(ctx.token_ids), _ptr(ctx.src_row),
+                           _ptr(ctx.prev_tokens), _ptr(ctx.positions), _ptr(ctx.seg_of_token), _ptr(ctx.cu_q),
+                           _ptr(ctx.state_slots), _ptr(last), _ptr(out), _ptr(keep), c_int(T), c_int(B), c_int(d),
+                           c_int(V), c_int(pair_table.shape[0] - 1), ctypes.c_longlong(mul_prev),
+                           ctypes.c_longlong(mul_cur), _stream()), "pair_embed")
+    return out
 
 
 def dual_norm_mix(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, ca: float, cb: float,
@@ -931,11 +1018,24 @@ def gated_group_norm(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, we
 # routed experts
 # ---------------------------------------------------------------------------------------------
 
+ROUTER_MODES = {"chosen": 0, "all": 1, "sigmoid": 2}
+
+
+def _router_mode(over_all) -> int:
+    """The kernels' number for a way of weighting the chosen experts: a name of ROUTER_MODES, or the older flag
+    (True = "all", False = "chosen")."""
+    if isinstance(over_all, str):
+        _check(over_all in ROUTER_MODES, f"unknown router mode {over_all!r}; known: {sorted(ROUTER_MODES)}")
+        return ROUTER_MODES[over_all]
+    return 1 if over_all else 0
+
+
 def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, weights: torch.Tensor,
-              over_all: bool = False, scale: float = 1.0) -> None:
+              over_all=False, scale: float = 1.0) -> None:
     """Per row of logits fp32 [T, >= experts]: the `top` experts with the largest logits (ids int32
-    [T, top]) and their weights fp32 [T, top]: the softmax over those logits alone, or (`over_all`) their
-    shares of the softmax over all experts divided by the sum of the chosen shares + 1e-20; times `scale`."""
+    [T, top]) and their weights fp32 [T, top]: the softmax over those logits alone ("chosen"), or (`over_all` True
+    or "all") their shares of the softmax over all experts divided by the sum of the chosen shares + 1e-20, or
+    ("sigmoid") the sigmoid of each chosen logit, not normalised; times `scale`."""
     _dev(logits, ids, weights)
     T = logits.shape[0]
     _check(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "router logits must be fp32 [T, >= E]")
@@ -944,7 +1044,7 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, ids: torch.Tensor, w
            "ids int32 [T, top], weights fp32 [T, top]")
     lib = load_library("moe")
     _ret(lib.sa_moe_route(_ptr(logits), c_int(logits.shape[1]), _ptr(ids), _ptr(weights), c_int(T), c_int(experts),
-                          c_int(top), c_int(1 if over_all else 0), c_float(scale), _stream()), "moe_route")
+                          c_int(top), c_int(_router_mode(over_all)), c_float(scale), _stream()), "moe_route")
 
 
 MOE_ROUTE_INSIDE = 16      # up to this many tokens the experts' call does the routing itself (one kernel less)
@@ -961,12 +1061,14 @@ def moe_wide_available(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                 yk: torch.Tensor, logits: Optional[torch.Tensor] = None,
-                weights: Optional[torch.Tensor] = None, over_all: bool = False, scale: float = 1.0,
-                gate: str = "silu", limit: float = 0.0) -> torch.Tensor:
+                weights: Optional[torch.Tensor] = None, over_all=False, scale: float = 1.0,
+                gate: str = "silu", limit: float = 0.0, weight_inputs: bool = False) -> torch.Tensor:
     """yk[t * top + k] = expert ids[t, k] applied to h[t]: down(gate(gate h, up h)), fp32 [T top, d], with
     one of GATES (silu(g) u unless said otherwise).
     w_gate, w_up [E, F, d], w_down [E, d, F] in h's dtype.  With `logits` (fp32 [T, >= E], at most
-    MOE_ROUTE_INSIDE tokens) `ids` and `weights` are made here as `moe_route` makes them (`over_all`, `scale`)."""
+    MOE_ROUTE_INSIDE tokens) `ids` and `weights` are made here as `moe_route` makes them (`over_all`, `scale`).
+    `weight_inputs`: expert ids[t, k] is applied to weights[t, k] * h[t] (the weight enters where the gate is applied,
+    gate and up being linear), for designs whose weights multiply the experts' inputs and not their outputs."""
     _dev(h, ids, w_gate, w_up, w_down, yk, logits, weights)
     T, d = h.shape
     top = ids.shape[1]
@@ -982,7 +1084,10 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
     tiles = int(lib.sa_moe_max_tiles(c_int(n), c_int(E)))
     ints = torch.empty(2 * E + 1 + n + 2 * tiles + 1, dtype=torch.int32, device=h.device)
     act = torch.empty((n, F), dtype=h.dtype, device=h.device)
-    if n > MOE_WIDE_MIN_ROWS and logits is None and moe_wide_available(h, w_gate, w_up, w_down):
+    if weight_inputs:
+        _check(weights is not None and weights.dtype == torch.float32 and weights.shape == (T, top)
+               and weights.is_contiguous(), "weights on the experts' inputs must be contiguous fp32 [T, top]")
+    if n > MOE_WIDE_MIN_ROWS and logits is None and not weight_inputs and moe_wide_available(h, w_gate, w_up, w_down):
         # prompt portions: the grouping here, the two products over tiles of 128 rows with both operands through LDS
         wide = load_library("gemm_mfma")
         rows = int(wide.sa_moe_wide_tile_rows())
@@ -1006,20 +1111,23 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
         ldz = logits.shape[1]
     _ret(lib.sa_moe_experts(_ptr(h), c_int(_code(h)), _ptr(ids), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(ints),
                             _ptr(act), _ptr(yk), c_int(T), c_int(top), c_int(E), c_int(d), c_int(F), _ptr(logits),
-                            c_int(ldz), _ptr(weights), c_int(1 if over_all else 0), c_float(scale), c_int(GATES[gate]),
-                            c_float(limit), _stream()), "moe_experts")
+                            c_int(ldz), _ptr(weights), c_int(_router_mode(over_all)), c_float(scale), c_int(GATES[gate]),
+                            c_float(limit), _ptr(weights if weight_inputs else None), _stream()), "moe_experts")
     return yk
 
 
-def moe_combine(yk: torch.Tensor, weights: torch.Tensor, shared: Optional[torch.Tensor],
+def moe_combine(yk: torch.Tensor, weights: Optional[torch.Tensor], shared: Optional[torch.Tensor],
                 logits: Optional[torch.Tensor], gate_col: int, y: torch.Tensor) -> torch.Tensor:
     """y[t] = sum_k weights[t, k] yk[t top + k] (+ sigmoid(logits[t, gate_col]) * shared[t]);
-    shared [T, d] or fp32 [parts, T, d]; logits None: the shared rows are added as they are."""
+    shared [T, d] or fp32 [parts, T, d]; logits None: the shared rows are added as they are; weights None: the
+    experts' rows are added as they are."""
     _dev(yk, weights, shared, logits, y)
-    T, top = weights.shape
-    d = y.shape[1]
-    _check(y.dtype == torch.float32 and y.shape == (T, d) and yk.shape == (T * top, d) and yk.dtype == torch.float32
-           and weights.dtype == torch.float32, "moe_combine: fp32 y [T, d], yk [T top, d], weights [T, top]")
+    T, d = y.shape
+    _check(T > 0 and yk.dim() == 2 and yk.shape[0] % T == 0, "moe_combine: yk must be [T top, d]")
+    top = yk.shape[0] // T
+    _check(y.dtype == torch.float32 and yk.shape == (T * top, d) and yk.dtype == torch.float32
+           and (weights is None or (weights.dtype == torch.float32 and weights.shape == (T, top))),
+           "moe_combine: fp32 y [T, d], yk [T top, d], weights [T, top]")
     parts, scode = 1, F32
     if shared is not None:
         if shared.dim() == 3:

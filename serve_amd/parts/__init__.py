@@ -3,4 +3,4 @@ from .base import (CacheTensor, LayerCache, ParamRequest, Part, PositionPart, Ro
                    StateRequest, TokenCacheRequest, kv_cache_request)
 from . import standard  # noqa: F401
 from . import postnorm, recurrent, latent, feedforward, normed_attention  # noqa: F401
-from . import gated_attention, linear_recurrent, parallel, token_input  # noqa: F401
+from . import gated_attention, linear_recurrent, parallel, token_input, rotary_attention  # noqa: F401

@@ -200,6 +200,7 @@ class Rotary:
     inv_freq: torch.Tensor          # fp32 [rot_dim / 2] on the device
     rot_dim: int
     adjacent_pairs: bool            # pair j = (2j, 2j + 1); else (j, j + rot_dim / 2)
+    magnitude: float = 1.0          # multiplies sine and cosine (a rotation that also stretches)
 
 
 class PositionPart(Part):

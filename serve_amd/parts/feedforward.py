@@ -15,7 +15,7 @@ from .standard import SwiGLU, _prepare_products
 
 
 class DenseFeedForward(Part):
-    """down(act(up x)), no biases; act = 'gelu_tanh' or 'silu'."""
+    """down(act(up x)), no biases; act = one of `ops.ACTIVATIONS` ('gelu_tanh', 'silu', 'relu_squared')."""
 
     graph_safe = True
 
@@ -47,25 +47,28 @@ class RoutedExperts(Part):
 
     `activation` / `limit`: another gate of `ops.GATES` in the experts (`shared_limit`: the shared expert's
     limit, if it differs).  `router_softmax="all"`: the weights are the chosen experts' shares of the softmax
-    over all experts, divided by their sum (+ 1e-20); `router_scale` multiplies the weights."""
+    over all experts, divided by their sum (+ 1e-20); `"sigmoid"`: the weights are the sigmoids of the chosen
+    logits as they are; `router_scale` multiplies the weights.  `weight_inputs`: a weight multiplies its expert's
+    input and not its output (the experts' outputs are then added as they are)."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, experts: int, top: int, expert_size: int,
                  shared_size: Optional[int] = None, shared_gate: bool = True, activation: str = "silu",
                  limit: float = 0.0, shared_limit: Optional[float] = None, router_softmax: str = "chosen",
-                 router_scale: float = 1.0):
+                 router_scale: float = 1.0, weight_inputs: bool = False):
         if not 0 < top <= experts:
             raise ValueError("top must be within the number of experts")
-        if router_softmax not in ("chosen", "all"):
-            raise ValueError("router_softmax must be 'chosen' or 'all'")
+        if router_softmax not in ops.ROUTER_MODES:
+            raise ValueError(f"router_softmax must be one of {sorted(ops.ROUTER_MODES)}")
         if activation not in ops.GATES:
             raise ValueError(f"unknown gate {activation!r}; known: {sorted(ops.GATES)}")
         self.hidden_size, self.experts, self.top, self.expert_size = int(hidden_size), int(experts), int(top), int(expert_size)
         self.shared_size = None if not shared_size else int(shared_size)
         self.shared_gate = bool(shared_gate) and self.shared_size is not None
         self.activation, self.limit = activation, float(limit)
-        self.over_all, self.router_scale = router_softmax == "all", float(router_scale)
+        self.over_all, self.router_scale = router_softmax, float(router_scale)      # (the router's mode, by name)
+        self.weight_inputs = bool(weight_inputs)
         self.shared = None
         if self.shared_size:
             self.shared = SwiGLU(self.hidden_size, self.shared_size, activation,
@@ -122,13 +125,15 @@ class RoutedExperts(Part):
         yk = torch.empty((T * self.top, d), dtype=torch.float32, device=dev)
         if T <= ops.MOE_ROUTE_INSIDE:
             ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, logits, weights, self.over_all,
-                            self.router_scale, self.activation, self.limit)                    # routes, too
+                            self.router_scale, self.activation, self.limit, self.weight_inputs)    # routes, too
         else:
             ops.moe_route(logits, self.experts, self.top, ids, weights, self.over_all, self.router_scale)
-            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, gate=self.activation, limit=self.limit)
+            ops.moe_experts(h, ids, self.w_gate, self.w_up, self.w_down, yk, weights=weights, gate=self.activation,
+                            limit=self.limit, weight_inputs=self.weight_inputs)
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         y = torch.empty((T, d), dtype=torch.float32, device=dev)
-        return ops.moe_combine(yk, weights, shared, logits if self.shared_gate else None, self.experts, y)
+        return ops.moe_combine(yk, None if self.weight_inputs else weights, shared,
+                               logits if self.shared_gate else None, self.experts, y)
 
 
 register_part("feed_forward", "dense", DenseFeedForward)

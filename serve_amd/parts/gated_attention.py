@@ -88,8 +88,8 @@ class GatedRotaryAttention(Part):
         if self.position is not None:
             self.position.load({}, rt)
             rot = self.position.rotary()
-            if rot is None or rot.adjacent_pairs:
-                raise ValueError("this attention takes a rotation of the pairs (i, i + rot/2), or no position part")
+            if rot is None or rot.adjacent_pairs or rot.magnitude != 1.0:
+                raise ValueError("this attention takes a plain rotation of the pairs (i, i + rot/2), or no position part")
             self.inv_freq, self.rot_dim = rot.inv_freq.contiguous(), int(rot.rot_dim)
             if self.rot_dim > self.dim:
                 raise ValueError(f"a rotation of {self.rot_dim} dims does not fit heads of {self.dim}")

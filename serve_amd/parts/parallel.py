@@ -6,6 +6,10 @@ over the model width, multiplied by a weight of their own and averaged:
 The two mixers are parts like any others (any registered mixer kinds); their tensors are named `left.*` and
 `right.*`, the two weights `left.out` and `right.out`.  At most one of the two may keep per-token cache; their
 per-request states lie one behind the other in the layer's state row.
+
+`ParallelResidual` (an arrangement) is the other kind of side by side: a mixer and a feed-forward behind ONE norm,
+
+    h = N(x) w;   x <- x + mixer(h) + ff(h)
 """
 from __future__ import annotations
 
@@ -96,4 +100,38 @@ class ParallelMixers(Part):
         return ops.dual_norm_mix(outs[0], outs[1], self.out_w["left"], self.out_w["right"], 0.5, 0.5, self.eps, out)
 
 
+class ParallelResidual:
+    """x <- x + mixer(h) + ffn(h), h = norm(x): one norm a layer, and both sublayers read its output.
+
+    As in the other arrangements the additions are folded into later kernels: the mixer's output joins the stream in
+    one pass of its own (`stream_add`), the feed-forward's is returned as what is still to be added and rides in the
+    next layer's norm.  A layer may have no feed-forward."""
+
+    PART_ROLES = {"mixer": "mixer", "ffn": "feed_forward", "norm": "norm"}
+    OPTIONAL_PARTS = ("ffn",)
+
+    def __init__(self, mixer, norm, ffn=None):
+        self.mixer, self.norm, self.ffn = mixer, norm, ffn
+
+    def cache_owner(self) -> Part:
+        return self.mixer
+
+    def parts(self) -> Dict[str, Part]:
+        out = {"mixer": self.mixer, "norm": self.norm}
+        if self.ffn is not None:
+            out["ffn"] = self.ffn
+        return out
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache: LayerCache,
+                writes_cache: bool = True) -> Optional[torch.Tensor]:
+        h = self.norm.forward(x, pending)
+        a = self.mixer.forward(h, ctx, cache, writes_cache)
+        if self.ffn is None:
+            return a
+        b = self.ffn.forward(h, ctx)
+        ops.stream_add(x, a)
+        return b
+
+
 register_part("mixer", "parallel", ParallelMixers)
+register_part("arrangement", "parallel_residual", ParallelResidual)

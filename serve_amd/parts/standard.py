@@ -69,8 +69,10 @@ def rope_inverse_frequencies(head_dim_rot: int, theta: float, scaling: Optional[
     if scaling is None:
         return f
     kind = scaling.get("rope_type", scaling.get("type", "llama3"))
+    if kind == "yarn":
+        return yarn_frequencies(head_dim_rot, theta, scaling)[0]
     if kind != "llama3":
-        raise ValueError(f"rope scaling {kind!r} is not supported (known: 'llama3')")
+        raise ValueError(f"rope scaling {kind!r} is not supported (known: 'llama3', 'yarn')")
     factor = float(scaling["factor"])
     low = float(scaling["low_freq_factor"])
     high = float(scaling["high_freq_factor"])
@@ -80,6 +82,33 @@ def rope_inverse_frequencies(head_dim_rot: int, theta: float, scaling: Optional[
     blended = (1 - smooth) * f / factor + smooth * f
     out = torch.where(wavelen < orig / high, f, torch.where(wavelen > orig / low, f / factor, blended))
     return out.float()
+
+
+def yarn_frequencies(rot_dim: int, theta: float, scaling: dict):
+    """(frequencies fp32 [rot_dim / 2], magnitude) of a rotation stretched to longer contexts by blending, per
+    pair, the plain frequency f_i = theta^(-2i/rot_dim) with f_i / factor:
+
+        turns(n) = rot_dim ln(original / (2 pi n)) / (2 ln theta)      the pair that makes n turns over `original` positions
+        lo = max(floor(turns(fast)), 0),  hi = min(ceil(turns(slow)), rot_dim - 1)
+        ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+        f_i' = f_i / factor * ramp_i + f_i (1 - ramp_i)
+
+    and sine and cosine are multiplied by 0.1 ln(factor) + 1.  Keys of `scaling`: factor, original, fast, slow.
+    Computed in float64 and rounded once."""
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    fast, slow = float(scaling["fast"]), float(scaling["slow"])
+    if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and theta > 1):
+        raise ValueError("yarn scaling needs positive factor, original, fast and slow, and a base above 1")
+    i = torch.arange(rot_dim // 2, dtype=torch.float64)
+    f = float(theta) ** (-2.0 * i / rot_dim)
+
+    def turns(n: float) -> float:
+        return rot_dim * math.log(original / (2.0 * math.pi * n)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(turns(fast)), 0)
+    hi = min(math.ceil(turns(slow)), rot_dim - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).float(), 0.1 * math.log(factor) + 1.0
 
 
 # largest angle (position * frequency, in radians) whose sine and cosine the bfloat16 kernels'
@@ -95,7 +124,8 @@ class RotaryPosition(PositionPart):
     (serve/hf_utils/convert_hf_checkpoint.py:115-118), which is `pairing="adjacent"`.
     `rot_dim < head_dim` leaves the remaining dims of every head as they are.  The part only
     says what the rotation is (`rotary()`); the attention's kernels carry it out, fused with
-    the projection or the cache write."""
+    the projection or the cache write.  `scaling` with `rope_type` "llama3" or "yarn" (see
+    `rope_inverse_frequencies`, `yarn_frequencies`); the latter also gives the rotation a magnitude."""
 
     graph_safe = True
 
@@ -117,7 +147,10 @@ class RotaryPosition(PositionPart):
                 raise ValueError(f"a context of {rt.max_context} tokens gives rotation angles up to {top:.3g} rad; "
                                  f"the bfloat16 kernels hold up to {ROTARY_MAX_ANGLE_REDUCED:.3g} "
                                  "(use dtype float32, or a shorter max_context)")
-        self._rotary = Rotary(f.to(rt.device), self.rot_dim, self.pairing == "adjacent")
+        magnitude = 1.0
+        if self.scaling is not None and self.scaling.get("rope_type", self.scaling.get("type")) == "yarn":
+            magnitude = yarn_frequencies(self.rot_dim, self.theta, self.scaling)[1]
+        self._rotary = Rotary(f.to(rt.device), self.rot_dim, self.pairing == "adjacent", magnitude)
 
     def rotary(self) -> Rotary:
         return self._rotary
@@ -176,6 +209,9 @@ class GQAAttention(Part):
         self.wo = tensors["o_proj.weight"]
         _prepare_products(rt, self.wqkv)
         self.position.load({}, rt)
+        rot = self.position.rotary()
+        if rot is not None and rot.magnitude != 1.0:
+            raise ValueError("this attention's kernels rotate without a magnitude; the kind 'rotary_attention' takes one")
         self._no_freq = torch.empty(0, dtype=torch.float32, device=rt.device)
 
     def _project_encode_store(self, h: torch.Tensor, ctx, cache: LayerCache, slots: Optional[torch.Tensor]):

@@ -8,7 +8,10 @@ row of the token, and x the stream after the layer's sublayers,
 The second table is the embedding part's (`embedding.side`); a layer reads the columns [offset, offset + dim).
 
 `PassVectors` (role `stream_input`, a part of the model): a table [rows, width] of which the run order adds one row to
-the stream before an entry runs.
+the stream before an entry runs (and, where the entry says so, the embedding's output once more).
+
+`PairEmbedding` (role `embedding`): the token's row plus a row of a second table chosen by a hash of the pair
+(previous token, token); the previous token of a request is per-request state.
 """
 from __future__ import annotations
 
@@ -18,7 +21,7 @@ import torch
 
 from .. import ops
 from ..registry import register_part
-from .base import NORMED_STREAM, ParamRequest, Part, Runtime, StepCost
+from .base import NORMED_STREAM, LayerCache, ParamRequest, Part, Runtime, StateRequest, StepCost
 from .linear import linear
 
 
@@ -84,13 +87,56 @@ class PassVectors(Part):
         self.rt = rt
         self.table = tensors["weight"].float().contiguous()          # the stream is fp32
 
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], row: int) -> Optional[torch.Tensor]:
-        """x += pending + table[row]; nothing is left to be added."""
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], row: int,
+                extra: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """x += pending + table[row] (+ extra, fp32 [T, width]); nothing is left to be added."""
         if not 0 <= row < self.rows:
             raise ValueError(f"pass vector {row} of {self.rows}")
-        ops.stream_add(x, pending, self.table[row], None)
+        ops.stream_add(x, pending, self.table[row], None, extra)
         return None
 
+
+class PairEmbedding(Part):
+    """x = E[token] + B[(previous token * mul_prev + token * mul_cur) mod buckets]; a sequence's first token takes
+    B's last row (B has buckets + 1 rows).  The previous token of a request's next portion is kept in a per-request
+    state row (`state_request`), read and replaced by the embedding's kernels on the device, so that portions cut
+    anywhere, and tokens that never reached the host, see the right row."""
+
+    graph_safe = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        if self.buckets <= 0 or self.mul_prev < 0 or self.mul_cur < 0:
+            raise ValueError("buckets must be positive, the multipliers not negative")
+        if max(self.mul_prev, self.mul_cur) * self.vocab_size >= 2 ** 62:
+            raise ValueError("the pair's hash must fit 64 bits")
+
+    def param_requests(self) -> List[ParamRequest]:
+        return [ParamRequest("weight", (self.vocab_size, self.hidden_size)),
+                ParamRequest("pairs", (self.buckets + 1, self.hidden_size))]
+
+    def state_request(self) -> StateRequest:
+        return StateRequest((1,), torch.int32)           # the request's latest token
+
+    def step_cost(self, tokens: int, context_before: int = 0) -> StepCost:
+        return StepCost(0, 0.0)                          # (gathered rows, as for the plain embedding)
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = tensors["weight"]
+        self.pairs = tensors["pairs"].to(self.weight.dtype).contiguous()
+
+    def forward(self, ctx, cache: LayerCache, keep: bool = False):
+        """fp32 [T, width]; with `keep` also a second copy of it, for whoever adds it to the stream again."""
+        T = ctx.token_ids.numel()
+        x = self.rt.empty((T, self.hidden_size), torch.float32)
+        copy = self.rt.empty((T, self.hidden_size), torch.float32) if keep else None
+        ops.pair_embed(self.weight, self.pairs, ctx, cache.state, x, self.mul_prev, self.mul_cur, copy)
+        return (x, copy) if keep else x
+
+
+register_part("embedding", "pair_embedding", PairEmbedding)
 
 register_part("token_input", "gated_side_embedding", GatedSideEmbedding)
 register_part("stream_input", "pass_vectors", PassVectors)

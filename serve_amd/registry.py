@@ -86,3 +86,4 @@ def _ensure_builtin() -> None:
         from .models import zozosun  # noqa: F401  (registers Zozosun)
         from .models import timopel  # noqa: F401  (registers Timopel)
         from .models import kotipel  # noqa: F401  (registers Kotipel)
+        from .models import robuvik  # noqa: F401  (registers Robuvik)
