@@ -62,8 +62,10 @@ def rotate(x: torch.Tensor, positions: torch.Tensor, f: torch.Tensor, magnitude:
     return out
 
 
-def embedding(tokens: List[int], embed: torch.Tensor, bigram: torch.Tensor, cfg: dict) -> torch.Tensor:
-    b = cfg["embedding"]["bigram"]
+def embedding(tokens: List[int], embed: torch.Tensor, bigram: Optional[torch.Tensor], cfg: dict) -> torch.Tensor:
+    b = (cfg.get("embedding") or {}).get("bigram")
+    if not b:
+        return embed[torch.tensor(tokens)]
     rows = []
     for p, t in enumerate(tokens):
         rows.append(b["buckets"] if p == 0 else (tokens[p - 1] * b["mul_prev"] + t * b["mul_cur"]) % b["buckets"])
@@ -176,7 +178,7 @@ def forward(model: dict, tokens: List[int], streams: Optional[list] = None) -> t
     """Logits [T, vocab] of a whole sequence; `streams` collects the residual stream after every layer run."""
     cfg, t = model["config"], model["tensors"]
     eps = cfg["norm"]["eps"]
-    x0 = embedding(tokens, t["embed"], t["bigram"], cfg)
+    x0 = embedding(tokens, t["embed"], t.get("bigram"), cfg)
     x = x0.clone()
     loop = cfg.get("loop")
     for i, pas in layer_passes(cfg):
