@@ -222,7 +222,7 @@ def report(engine, cfg, steps: int, warmup: int, make_engine=None) -> int:
 
 
 def designs(args) -> int:
-    """`--designs`: prefill and decode throughput of the Zozosun, Timopel and Kotipel shapes, each beside the Llama shape of the same
+    """`--designs`: prefill and decode throughput of the Zozosun, Timopel, Kotipel and Robuvik shapes, each beside the Llama shape of the same
     width, depth, vocabulary and feed-forward width (serve_amd.benchmark.DESIGN_PAIRS), random weights.  One
     JSON line per model: tokens/s of a 2,048-token prompt, and of decode steps at batch 1, 8 and 64 with
     contexts around `--context`; with the bytes a decode step streams and the flops of the prompt as the
@@ -292,7 +292,7 @@ def main() -> int:
                     help="print a table instead of the JSON line: decode at batch 1, 8 and 64 and the prefill, each "
                     "with its bytes or flops, as a share of the published peaks and of ceilings measured here")
     ap.add_argument("--designs", action="store_true",
-                    help="measure the Zozosun, Timopel and Kotipel shapes beside Llama shapes of equal size instead (prefill of 2,048 tokens, "
+                    help="measure the Zozosun, Timopel, Kotipel and Robuvik shapes beside Llama shapes of equal size instead (prefill of 2,048 tokens, "
                     "decode at batch 1, 8 and 64); one JSON line per model; --shape picks one pair")
     args = ap.parse_args()
     if args.gpus != 1:

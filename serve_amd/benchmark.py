@@ -128,8 +128,37 @@ SHAPES.update({
     "kotipel-2k": _kotipel_shape(2048, 32768, 6, (2, 4, 2), 32, 8, 64, 16, 64, 128, 64, 1, 8192, 256),
     "kotipel-4k": _kotipel_shape(4096, 32768, 3, (1, 2, 2), 32, 8, 128, 16, 128, 256, 128, 8, 14336, 256),
 })
+
+
+def _robuvik_shape(width: int, vocab: int, layers: int, loop, heads: int, kv_heads: int, head: int, window: int,
+                   q_rank: int, ff: int, experts: int, top: int, expert_ff: int, shared_ff: int, buckets: int):
+    """A Robuvik shape at the sizes of a real model's layers: in turn an attention layer (`heads` on `kv_heads` heads
+    of `head`, all dims rotated with stretched frequencies, a window, biases, a sink) with a dense feed-forward of
+    `ff`, and a latent-attention layer (`heads` heads of 64 + 32 rotated dims over a latent of 96: a cache row as
+    wide as the matrix-core attention's widest head; queries through a latent of `q_rank`) with routed experts and a
+    shared one; `loop` = (start, stop, times); a pair table of `buckets` rows."""
+    from .config.kotipel import LoopConfig
+    from .config.robuvik import (BigramConfig, DenseConfig, ExpertsConfig, LatentAttentionConfig, RobuvikConfig,
+                                 RobuvikLayerConfig, RotConfig, WindowAttentionConfig, YarnScaling)
+    yarn = YarnScaling(4.0, 2048.0, 32.0, 1.0)
+    att = WindowAttentionConfig(heads, kv_heads, head, head, head ** -0.5, RotConfig(500000.0, head, yarn), window)
+    lat = LatentAttentionConfig(heads, 64, 32, 64, 96, q_rank, 96 ** -0.5, RotConfig(1.0e6, 32, yarn))
+    moe = ExpertsConfig(experts, top, expert_ff, shared_ff)
+    return RobuvikConfig(vocab=vocab, width=width, eps=1e-5, bigram=BigramConfig(buckets, 31, 7), loop=LoopConfig(*loop),
+                         layers=tuple(RobuvikLayerConfig(att, DenseConfig(ff)) if i % 2 == 0 else RobuvikLayerConfig(lat, moe)
+                                      for i in range(layers)))
+
+
+# Robuvik at the same two widths, vocabularies, attention head shapes and dense feed-forward widths (its experts as
+# Zozosun's and Timopel's); with the layers that run twice it has as many layer runs as the Llama shapes have layers
+SHAPES.update({
+    "robuvik-tiny": _robuvik_shape(64, 512, 2, (0, 2, 2), 4, 2, 16, 24, 32, 128, 4, 2, 32, 64, 251),
+    "robuvik-2k": _robuvik_shape(2048, 32768, 6, (2, 4, 2), 32, 8, 64, 1024, 512, 8192, 32, 4, 1024, 2048, 65521),
+    "robuvik-4k": _robuvik_shape(4096, 32768, 3, (1, 2, 2), 32, 8, 128, 1024, 1024, 14336, 64, 6, 1536, 3072, 65521),
+})
 DESIGN_PAIRS = (("zozosun-2k", "llama-2k"), ("zozosun-4k", "llama-4k"), ("timopel-2k", "llama-2k"),
-                ("timopel-4k", "llama-4k"), ("kotipel-2k", "llama-2k"), ("kotipel-4k", "llama-4k"))
+                ("timopel-4k", "llama-4k"), ("kotipel-2k", "llama-2k"), ("kotipel-4k", "llama-4k"),
+                ("robuvik-2k", "llama-2k"), ("robuvik-4k", "llama-4k"))
 
 
 def generate_requests(input_length: int, output_length: int, num_sequences: int, vocab_size: int,

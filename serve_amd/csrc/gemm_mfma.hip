@@ -65,6 +65,7 @@ struct MoeTileArgs {
   const int* tile_row0;
   const int* num_tiles;
   int top;
+  const float* in_wts;      // MOE 1: fp32 [token * top + k], multiplies gate and up sums before the gate (null: not)
 };
 
 // silu(g) u with the fast exponential, as the plain SwiGLU feed-forward has always been computed; any other gate
@@ -763,7 +764,11 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
   for (int mt = 0; mt < MW; ++mt) {
     int m = m0 + (mw * MW + mt) * 16 + c;
     if (m >= M) continue;
-    if constexpr (MOE == 1) m += moe_row0;                 // the grouped row
+    float in_w = 1.f;                                      // (a weight on the expert's input: gate and up are linear in it)
+    if constexpr (MOE == 1) {
+      m += moe_row0;                                       // the grouped row
+      if (SWIGLU && ma.in_wts) in_w = ma.in_wts[ma.perm[m]];
+    }
     if constexpr (MOE == 2) m = ma.perm[moe_row0 + m];     // (token, k)
 #pragma unroll
     for (int nt = 0; nt < (SWIGLU ? NT / 2 : NT); ++nt) {
@@ -772,8 +777,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16_t* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if (SWIGLU) {
-          const float gt = acc[mt][nt][r];
-          o[r] = gated(gt, acc[mt][SWIGLU ? nt + NT / 2 : nt][r], qa);
+          const float gt = acc[mt][nt][r] * in_w;
+          o[r] = gated(gt, acc[mt][SWIGLU ? nt + NT / 2 : nt][r] * in_w, qa);
         } else {
           o[r] = acc[mt][nt][r];
         }
@@ -1143,17 +1148,18 @@ extern "C" int sa_moe_wide_tile_rows() { return MOE_WIDE_ROWS; }
 // sa_moe_experts with products = 0; max_tiles: the grid's worst case, rows / tile_rows + E).  bf16; d and F
 // multiples of 64 (whole stages of K).
 //   gate/up: h [T, d] gathered by perm / top, Wgu [2, E, F, d] -> act [rows, F] = gate(gate, up)
+//            (in_wts, fp32 [T top] or null: both sums times the row's weight first, for weights on the experts' inputs)
 //   down:    act [rows, F], Wd [E, d, F] -> yk [T top, d] fp32 at row perm[r]
 extern "C" int sa_moe_wide(const void* h, const void* Wgu, const void* Wd, void* act, float* yk, int E, int d, int F,
                            int max_tiles, const int* offsets, const int* perm, const int* tile_expert,
                            const int* tile_row0, const int* num_tiles, int top, int gate_kind, float gate_limit,
-                           hipStream_t stream) {
+                           const float* in_wts, hipStream_t stream) {
   if (E <= 0 || d <= 0 || F <= 0 || (d & 63) || (F & 63) || top <= 0) return SA_ERR_ARG;
   if (gate_kind < 0 || gate_kind >= SA_GATE_KINDS || (long long)E * F > 0x7fffffffLL) return SA_ERR_ARG;
   QkvRopeArgs qa = {};
   qa.gate_kind = gate_kind;
   qa.gate_limit = gate_limit;
-  const MoeTileArgs ma = {offsets, perm, tile_expert, tile_row0, num_tiles, top};
+  const MoeTileArgs ma = {offsets, perm, tile_expert, tile_row0, num_tiles, top, in_wts};
   int rc = launch_wide_moe<bf16_t, EPI_SWIGLU, 1>(h, Wgu, act, F, d, E * F, max_tiles, qa, ma, stream);
   if (rc != 0) return rc;
   return launch_wide_moe<float, EPI_PLAIN, 2>(act, Wd, yk, d, F, 0, max_tiles, qa, ma, stream);

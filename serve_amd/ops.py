@@ -1087,7 +1087,7 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
     if weight_inputs:
         _check(weights is not None and weights.dtype == torch.float32 and weights.shape == (T, top)
                and weights.is_contiguous(), "weights on the experts' inputs must be contiguous fp32 [T, top]")
-    if n > MOE_WIDE_MIN_ROWS and logits is None and not weight_inputs and moe_wide_available(h, w_gate, w_up, w_down):
+    if n > MOE_WIDE_MIN_ROWS and logits is None and moe_wide_available(h, w_gate, w_up, w_down):
         # prompt portions: the grouping here, the two products over tiles of 128 rows with both operands through LDS
         wide = load_library("gemm_mfma")
         rows = int(wide.sa_moe_wide_tile_rows())
@@ -1100,7 +1100,7 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, w_gate: torch.Tensor, w_up: 
         _ret(wide.sa_moe_wide(_ptr(h), _ptr(w_gate), _ptr(w_down), _ptr(act), _ptr(yk), c_int(E), c_int(d), c_int(F),
                               c_int(-(-n // rows) + E), c_void_p(offsets), c_void_p(perm), c_void_p(tile_expert),
                               c_void_p(tile_row0), c_void_p(num_tiles), c_int(top), c_int(GATES[gate]), c_float(limit),
-                              _stream()), "moe_wide")
+                              _ptr(weights if weight_inputs else None), _stream()), "moe_wide")
         return yk
     ldz = 0
     if logits is not None:
