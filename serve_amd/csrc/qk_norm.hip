@@ -471,6 +471,132 @@ __global__ __launch_bounds__(256) void bias_rope_kv_write_kernel(
   v_pages[(((size_t)page * Hk + g) * Dp + i) * page_size + off] = out;
 }
 
+// The same for bf16 with pairs (j, j + rot / 2), rot % 16 == 0 and D, Dv, Dp and the row stride multiples of 8, from
+// 16-byte aligned arrays: 16-byte vectors, `tpb` (1, 2, 4 or 8) consecutive tokens a block.  A thread takes eight dims of
+// one head of one token: eight pairs (two loads, two stores) in the rotated part's first half, a plain copy behind the
+// rotated part, zeros in the padding.  The values go through LDS: read as rows of tokens, written so that neighbouring
+// lanes hold neighbouring tokens of one dim, which in the transposed page are neighbouring addresses when the tokens'
+// slots are (a prompt portion's are).
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    f[2 * k] = bf16_bits_to_float(w[k] & 0xffffu);
+    f[2 * k + 1] = bf16_bits_to_float(w[k] >> 16);
+  }
+}
+
+__device__ __forceinline__ uint4 pack8(const float* f) {
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    w[k] = (uint32_t)float_to_bf16_bits(f[2 * k]) | ((uint32_t)float_to_bf16_bits(f[2 * k + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__device__ __forceinline__ void add8(float* f, const float* __restrict__ b) {
+  if (!b) return;
+  const float4 b0 = *reinterpret_cast<const float4*>(b), b1 = *reinterpret_cast<const float4*>(b + 4);
+  f[0] += b0.x; f[1] += b0.y; f[2] += b0.z; f[3] += b0.w;
+  f[4] += b1.x; f[5] += b1.y; f[6] += b1.z; f[7] += b1.w;
+}
+
+__global__ __launch_bounds__(1024) void bias_rope_kv_write_vec_kernel(
+    const bf16_t* __restrict__ qkv, long long row_stride, bf16_t* __restrict__ q_out, const int* __restrict__ positions,
+    const int* __restrict__ slot, bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages,
+    const float* __restrict__ bias, const float* __restrict__ freq, int rot, float magnitude, int T, int Hq, int Hk, int D,
+    int Dv, int Dp, int page_size, int tpb) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char brk_lds[];
+  const int t0 = blockIdx.x * tpb;
+  const int nt = min(tpb, T - t0);
+  const int half = rot >> 1;
+  const int cph = Dp >> 3;                                   // chunks of eight dims a head
+  const int units = Hq + (slot ? Hk : 0);
+  const int per_token = units * cph;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  for (int idx = threadIdx.x; idx < nt * per_token; idx += blockDim.x) {
+    const int i = idx / per_token;
+    const int rem = idx - i * per_token;
+    const int u = rem / cph;
+    const int j0 = (rem - u * cph) * 8;
+    if (j0 >= half && j0 < rot) continue;                    // (the second halves of the pairs: their partners write them)
+    const int t = t0 + i;
+    const bool is_q = u < Hq;
+    const int g = is_q ? u : u - Hq;
+    bf16_t* dst;
+    if (is_q) {
+      dst = q_out + ((size_t)t * Hq + g) * Dp;
+    } else {
+      const int s = slot[t];
+      if (s < 0) continue;
+      const int page = s / page_size;
+      dst = k_pages + (((size_t)page * Hk + g) * page_size + (s - page * page_size)) * Dp;
+    }
+    if (j0 >= D) {
+      *reinterpret_cast<uint4*>(dst + j0) = zero;
+      continue;
+    }
+    const size_t col = (is_q ? 0 : (size_t)Hq * D) + (size_t)g * D;
+    const bf16_t* x = qkv + (size_t)t * row_stride + col;
+    const float* b = bias ? bias + col : nullptr;
+    float lo[8];
+    unpack8(*reinterpret_cast<const uint4*>(x + j0), lo);
+    add8(lo, b ? b + j0 : nullptr);
+    if (j0 >= rot) {
+      *reinterpret_cast<uint4*>(dst + j0) = pack8(lo);
+      continue;
+    }
+    float hi[8];
+    unpack8(*reinterpret_cast<const uint4*>(x + half + j0), hi);
+    add8(hi, b ? b + half + j0 : nullptr);
+    const float pos = (float)positions[t];
+    const float4 f0 = *reinterpret_cast<const float4*>(freq + j0), f1 = *reinterpret_cast<const float4*>(freq + j0 + 4);
+    const float fr[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
+    float o0[8], o1[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float sn, cs;
+      sincos_reduced(pos * fr[k], &sn, &cs);
+      sn *= magnitude;
+      cs *= magnitude;
+      o0[k] = lo[k] * cs - hi[k] * sn;
+      o1[k] = hi[k] * cs + lo[k] * sn;
+    }
+    *reinterpret_cast<uint4*>(dst + j0) = pack8(o0);
+    *reinterpret_cast<uint4*>(dst + half + j0) = pack8(o1);
+  }
+  if (!slot) return;
+  // values (with their bias): rows of tokens into LDS (16 bytes of padding a row spread the tokens over the banks) ...
+  const int HD = Hk * Dv;
+  const int stride = HD + 8;                                  // elements
+  uint16_t* tile = reinterpret_cast<uint16_t*>(brk_lds);
+  const int vecs = HD >> 3;
+  const size_t vcol = (size_t)(Hq + Hk) * D;
+  for (int idx = threadIdx.x; idx < nt * vecs; idx += blockDim.x) {
+    const int i = idx / vecs;
+    const int e0 = (idx - i * vecs) * 8;
+    uint4 v = *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + i) * row_stride + vcol + e0);
+    if (bias) {
+      float f[8];
+      unpack8(v, f);
+      add8(f, bias + vcol + e0);
+      v = pack8(f);
+    }
+    *reinterpret_cast<uint4*>(tile + i * stride + e0) = v;
+  }
+  __syncthreads();
+  // ... and out again with the token as the fastest index, every head padded with zeros up to Dp
+  const int i = threadIdx.x & (tpb - 1);
+  const int s = i < nt ? slot[t0 + i] : -1;
+  if (s < 0) return;
+  const int page = s / page_size;
+  bf16_t* vp = v_pages + (size_t)page * Hk * Dp * page_size + (s - page * page_size);
+  for (int e = threadIdx.x / tpb; e < Hk * Dp; e += blockDim.x / tpb) {
+    const int g = e / Dp, d = e - g * Dp;
+    vp[(size_t)e * page_size].v = d < Dv ? tile[i * stride + g * Dv + d] : (uint16_t)0;
+  }
+}
+
 extern "C" int sa_bias_rope_kv_write(const void* qkv, long long row_stride, void* q_out, int act_dtype,
                                      const int* positions, const int* slot, void* k_pages, void* v_pages,
                                      const float* bias, const float* freq, int rot, int adjacent, float magnitude, int T,
@@ -481,6 +607,21 @@ extern "C" int sa_bias_rope_kv_write(const void* qkv, long long row_stride, void
   if (row_stride < (long long)Hq * D + (long long)Hk * (D + Dv) || (slot && (!k_pages || !v_pages)) || rot < 0 || rot % 2 ||
       rot > D || (rot > 0 && !freq))
     return SA_ERR_ARG;
+  int tpb = T >= 1024 ? 8 : (T >= 512 ? 4 : (T >= 256 ? 2 : 1));
+  while (tpb > 1 && (size_t)tpb * ((size_t)Hk * Dv + 8) * 2 > 65536) tpb >>= 1;   // the values' tile has to fit LDS
+  const size_t tile_bytes = (size_t)tpb * ((size_t)Hk * Dv + 8) * 2;
+  const bool aligned = !(((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages | (uintptr_t)bias |
+                          (uintptr_t)freq) & 15);
+  if (act_dtype == SA_BF16 && !adjacent && (rot & 15) == 0 && !((D | Dv | Dp) & 7) && !(row_stride & 7) && aligned &&
+      tile_bytes <= 65536) {
+    const long long items = (long long)tpb * (Hq + (slot ? Hk : 0)) * (Dp >> 3);
+    const int vthreads = (int)(items >= 1024 ? 1024 : (items <= 256 ? 256 : (items + 63) / 64 * 64));
+    hipLaunchKernelGGL(bias_rope_kv_write_vec_kernel, dim3((T + tpb - 1) / tpb), dim3(vthreads), slot ? tile_bytes : 0,
+                       stream, (const bf16_t*)qkv, row_stride, (bf16_t*)q_out, positions, slot, (bf16_t*)k_pages,
+                       (bf16_t*)v_pages, bias, freq, rot, magnitude, T, Hq, Hk, D, Dv, Dp, page_size, tpb);
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
   const int threads = 256;
   const long long qk_blocks = ((long long)T * (Hq + (slot ? Hk : 0)) * Dp + threads - 1) / threads;
   const long long v_blocks = slot ? ((long long)T * Hk * Dp + threads - 1) / threads : 0;

@@ -356,18 +356,24 @@ def test_pair_embedding_over_steps(dtype, d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,Dv,Dp,rot,adjacent", [(4, 2, 32, 16, 32, 16, False), (6, 1, 24, 40, 48, 24, False),
-                                                       (3, 3, 10, 7, 16, 4, True), (2, 1, 136, 24, 144, 64, False),
-                                                       (2, 2, 16, 16, 16, 0, False), (5, 5, 8, 8, 16, 8, True)])
-def test_bias_rope_kv_write(dtype, H, G, D, Dv, Dp, rot, adjacent):
+@pytest.mark.parametrize("H,G,D,Dv,Dp,rot,adjacent,T", [
+    (4, 2, 32, 16, 32, 16, False, 11), (6, 1, 24, 40, 48, 24, False, 11), (3, 3, 10, 7, 16, 4, True, 11),
+    (2, 1, 136, 24, 144, 64, False, 11), (2, 2, 16, 16, 16, 0, False, 11), (5, 5, 8, 8, 16, 8, True, 11),
+    (4, 2, 32, 16, 32, 16, False, 300), (8, 2, 64, 64, 64, 64, False, 1100), (2, 1, 48, 40, 48, 32, False, 600)])
+def test_bias_rope_kv_write(dtype, H, G, D, Dv, Dp, rot, adjacent, T):
+    """Both kernels (an element a thread; for bfloat16 at sizes that are multiples of 8, eight dims a thread and the
+    values through LDS, with 1, 2, 4 and 8 tokens a workgroup), with and without biases, with slots that store nothing."""
     from serve_amd import ops
-    T, page, P = 11, 4, 6
-    g = torch.Generator().manual_seed(H * D + rot)
+    page = 4
+    P = (T + 30) // page + 2
+    g = torch.Generator().manual_seed(H * D + rot + T)
     cols = H * D + G * (D + Dv)
-    z = torch.randn(T, cols + 5, generator=g).to(dtype).cuda()                 # (rows wider than what is read)
+    z = torch.randn(T, cols + (8 if H % 2 == 0 else 5), generator=g).to(dtype).cuda()       # (rows wider than what is read)
     bias = torch.randn(cols, generator=g).cuda()
-    pos = torch.tensor([0, 1, 2, 3, 40, 41, 42, 300, 7, 8, 9], dtype=torch.int32, device="cuda")
-    slots = torch.tensor([0, 1, 2, 3, 20, 21, 22, -1, 9, 10, 11], dtype=torch.int32, device="cuda")
+    pos_l = [0, 1, 2, 3, 40, 41, 42, 300, 7, 8, 9] if T == 11 else [(5 * t) % 310 for t in range(T)]
+    slot_l = [0, 1, 2, 3, 20, 21, 22, -1, 9, 10, 11] if T == 11 else [-1 if t % 97 == 5 else t + 12 for t in range(T)]
+    pos = torch.tensor(pos_l, dtype=torch.int32, device="cuda")
+    slots = torch.tensor(slot_l, dtype=torch.int32, device="cuda")
     f, mag = (rp.rotary_frequencies(rot, 100.0, {"factor": 3.0, "original": 16.0, "fast": 4.0, "slow": 1.0})
               if rot else (torch.zeros(0, dtype=torch.float64), 1.0))
     inv = f.float().cuda()
@@ -387,16 +393,18 @@ def test_bias_rope_kv_write(dtype, H, G, D, Dv, Dp, rot, adjacent):
         tol = dict(atol=1e-4, rtol=2e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=2e-2)
         qq = q.view(T, H, Dp).double().cpu()
         assert torch.allclose(qq[..., :D], wq, **tol) and (qq[..., D:] == 0).all()
-        for t in range(T):
-            s = int(slots[t])
-            if s < 0:
-                continue
-            kk = k_pages[s // page, :, s % page].double().cpu()
-            vv = v_pages[s // page, :, :, s % page].double().cpu()
-            assert torch.allclose(kk[:, :D], wk[t], **tol) and (kk[:, D:] == 0).all()
-            assert torch.allclose(vv[:, :Dv], wv[t], **tol) and (vv[:, Dv:] == 0).all()
-        # the slot of the token that stores nothing, and slots nobody named, are untouched
-        assert all((k_pages[p] == 9).all() and (v_pages[p] == 9).all() for p in (1, 3, 4))
+        stored = [t for t in range(T) if slot_l[t] >= 0]
+        st = torch.tensor([slot_l[t] for t in stored])
+        kk = k_pages.double().cpu()[st // page, :, st % page]                    # [n, G, Dp]
+        vv = v_pages.double().cpu()[st // page, :, :, st % page]                 # [n, G, Dp]
+        assert torch.allclose(kk[..., :D], wk[stored], **tol) and (kk[..., D:] == 0).all()
+        assert torch.allclose(vv[..., :Dv], wv[stored], **tol) and (vv[..., Dv:] == 0).all()
+        # slots that nobody named are untouched
+        used = torch.zeros(P * page, dtype=torch.bool)
+        used[st] = True
+        free = (~used).nonzero()[:, 0]
+        assert (k_pages.cpu()[free // page, :, free % page] == 9).all()
+        assert (v_pages.cpu()[free // page, :, :, free % page] == 9).all()
         q2 = torch.empty_like(q)
         ops.bias_rope_kv_write(z, q2, pos, None, None, None, bias if with_bias else None, inv if rot else None, rot,
                                adjacent, mag, H, G, D, Dv)
