@@ -285,3 +285,53 @@ extern "C" int sa_activation(void* a, int act_dtype, long long n, int kind, hipS
   SA_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// An element-wise output gate: a[i] *= sigmoid(g[i]), in place, a and g of one shape and dtype.
+// ---------------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void sigmoid_mul_kernel(TA* __restrict__ a, const TA* __restrict__ g, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    a[i] = from_float<TA>(to_float(a[i]) / (1.f + expf(-to_float(g[i]))));
+}
+
+// the same, eight bf16 values a thread in 16-byte vectors (n % 8 == 0, 16-byte aligned)
+__global__ __launch_bounds__(256) void sigmoid_mul_bf16x8_kernel(bf16_t* __restrict__ a, const bf16_t* __restrict__ g,
+                                                                 size_t groups) {
+  for (size_t gi = (size_t)blockIdx.x * blockDim.x + threadIdx.x; gi < groups; gi += (size_t)gridDim.x * blockDim.x) {
+    const uint4 av = *reinterpret_cast<const uint4*>(a + gi * 8);
+    const uint4 gv = *reinterpret_cast<const uint4*>(g + gi * 8);
+    const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, gw[4] = {gv.x, gv.y, gv.z, gv.w};
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float r0 = bf16_bits_to_float(aw[k] & 0xffffu) / (1.f + expf(-bf16_bits_to_float(gw[k] & 0xffffu)));
+      const float r1 = bf16_bits_to_float(aw[k] >> 16) / (1.f + expf(-bf16_bits_to_float(gw[k] >> 16)));
+      w[k] = (uint32_t)float_to_bf16_bits(r0) | ((uint32_t)float_to_bf16_bits(r1) << 16);
+    }
+    *reinterpret_cast<uint4*>(a + gi * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+extern "C" int sa_sigmoid_mul(void* a, const void* g, int act_dtype, long long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (!a || !g) return SA_ERR_ARG;
+  if (act_dtype == SA_BF16 && (n & 7) == 0 && (((uintptr_t)a | (uintptr_t)g) & 15) == 0) {
+    long long vb = (n / 8 + 255) / 256;
+    if (vb > 65536) vb = 65536;
+    hipLaunchKernelGGL(sigmoid_mul_bf16x8_kernel, dim3((unsigned)vb), dim3(256), 0, stream, (bf16_t*)a, (const bf16_t*)g,
+                       (size_t)(n / 8));
+    SA_LAUNCH_CHECK();
+    return 0;
+  }
+  long long blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  dim3 grid((unsigned)blocks), block(256);
+  if (act_dtype == SA_F32)
+    hipLaunchKernelGGL(sigmoid_mul_kernel<float>, grid, block, 0, stream, (float*)a, (const float*)g, (size_t)n);
+  else if (act_dtype == SA_BF16)
+    hipLaunchKernelGGL(sigmoid_mul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, (const bf16_t*)g, (size_t)n);
+  else return SA_ERR_UNSUPPORTED;
+  SA_LAUNCH_CHECK();
+  return 0;
+}

@@ -459,6 +459,16 @@ def activation(a: torch.Tensor, kind: str) -> torch.Tensor:
     return a
 
 
+def sigmoid_mul(a: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """a *= sigmoid(g) in place, element by element (an output gate); a and g contiguous, of one shape and dtype."""
+    _dev(a, g)
+    _check(a.shape == g.shape and a.dtype == g.dtype and a.is_contiguous() and g.is_contiguous(),
+           "the gate's logits must have the shape and dtype of what they gate, both contiguous")
+    lib = load_library("sublayer")
+    _ret(lib.sa_sigmoid_mul(_ptr(a), _ptr(g), c_int(_code(a)), ctypes.c_longlong(a.numel()), _stream()), "sigmoid_mul")
+    return a
+
+
 # ---------------------------------------------------------------------------------------------
 # gated delta rule
 # ---------------------------------------------------------------------------------------------

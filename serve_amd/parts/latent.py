@@ -156,8 +156,7 @@ class LatentAttention(Part):
         o = self.rt.empty((T, H * self.vdim))
         ops.head_linear(attn, H * D, D, self.w_uv, o, H * self.vdim, self.vdim, T)
         if self.out_gate:
-            # an element-wise gate is a gate per head over heads of one element
-            ops.head_gate(o, linear(h, self.w_g), 0, H * self.vdim)
+            ops.sigmoid_mul(o, linear(h, self.w_g))
         return linear(o, self.wo, partial_ok=True)
 
 

@@ -465,7 +465,7 @@ def test_experts_weighted_on_their_inputs_by_sigmoid_scores(dtype, T, E, top, d,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_stream_add_with_a_second_array_and_the_squared_relu(dtype):
+def test_stream_add_with_a_second_array_the_squared_relu_and_the_output_gate(dtype):
     from serve_amd import ops
     g = torch.Generator().manual_seed(1)
     for T, d in ((3, 50), (70, 64), (5, 2304)):
@@ -483,6 +483,10 @@ def test_stream_add_with_a_second_array_and_the_squared_relu(dtype):
         a = torch.randn(3, n, generator=g).to(dtype).cuda()
         want = (a.float().clamp_min(0) ** 2).to(dtype)
         assert torch.equal(ops.activation(a.clone(), "relu_squared"), want)
+        gate = torch.randn(3, n, generator=g).to(dtype).cuda()
+        want = (a.float() * torch.sigmoid(gate.float())).to(dtype)
+        assert torch.allclose(ops.sigmoid_mul(a.clone(), gate).float(), want.float(), rtol=1e-2 if dtype == torch.bfloat16 else 1e-6,
+                              atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
