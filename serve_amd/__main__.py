@@ -104,7 +104,7 @@ def _random_model(argv) -> int:
     ap = argparse.ArgumentParser(prog="python -m serve_amd random-model")
     ap.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
     g = ap.add_mutually_exclusive_group(required=True)
-    g.add_argument("--shape", "--preset", dest="shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b, zozosun-tiny, zozosun-2k, timopel-tiny, timopel-2k, ...)")
+    g.add_argument("--shape", "--preset", dest="shape", help="a named shape (tiny, tiny-a, tiny-b, llama-1b, llama-3b, llama-8b, zozosun-tiny, zozosun-2k, timopel-tiny, timopel-2k, kotipel-tiny, robuvik-tiny, ...)")
     g.add_argument("--config", help="a config.json to take the sizes from")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--weight-dtype", choices=["bfloat16", "float32"], default="bfloat16",

@@ -11,6 +11,7 @@ The models differ in every size and option:
       rotation, dense), (latent attention with a plain rotation, experts top 3 of 3)
   RC  width 50 (no multiple of 8), vocabulary 101; both layers run three times; 3 heads on 3, keys 10 / values 7, 4
       rotated dims, a window of 33; latent attention 2 heads of 6 + 4, values 5, latents 9 / 7; experts of width 9
+  RE  RB with its first two layers run twice (a loop without a pair table)
   RD  sizes above what the matrix-core attention takes: keys 136 / values 24; a latent row of 200 + 16; a single layer
       that runs twice between two that run once
 """
@@ -54,7 +55,10 @@ RD = RobuvikConfig(vocab=120, width=64, eps=1e-5, bigram=BigramConfig(1021, 31, 
     L(ATT(2, 2, 136, 24, 0.1, None, 7), ExpertsConfig(2, 1, 16, None)),
 ))
 
-MODELS = {"RA": (RA, 3), "RB": (RB, 4), "RC": (RC, 5), "RD": (RD, 6)}
+# RB with its first two layers run twice: passes that add the output of an embedding without a pair table
+RE = RobuvikConfig(vocab=RB.vocab, width=RB.width, eps=RB.eps, bigram=None, loop=LoopConfig(0, 2, 2), layers=RB.layers)
+
+MODELS = {"RA": (RA, 3), "RB": (RB, 4), "RC": (RC, 5), "RD": (RD, 6), "RE": (RE, 7)}
 
 # tables and the output matrix at a scale at which the stream and the logits are of order one
 BASE = {r"^embed$": 40.0, r"^bigram$": 25.0, r"^head$": 6.0, r"^loop\.step$": 2.0}

@@ -56,7 +56,7 @@ def test_prompt_then_token_by_token(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("name", NAMES + ["RE"])
 def test_portions_of_changing_size(tmp_path, name, dtype):
     folder = rm.make_folder(tmp_path, name)
     engine = rm.engine_for(folder, dtype)
