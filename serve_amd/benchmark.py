@@ -144,7 +144,7 @@ def _robuvik_shape(width: int, vocab: int, layers: int, loop, heads: int, kv_hea
     att = WindowAttentionConfig(heads, kv_heads, head, head, head ** -0.5, RotConfig(500000.0, head, yarn), window)
     lat = LatentAttentionConfig(heads, 64, 32, 64, 96, q_rank, 96 ** -0.5, RotConfig(1.0e6, 32, yarn))
     moe = ExpertsConfig(experts, top, expert_ff, shared_ff)
-    return RobuvikConfig(vocab=vocab, width=width, eps=1e-5, bigram=BigramConfig(buckets, 31, 7), loop=LoopConfig(*loop),
+    return RobuvikConfig(vocab=vocab, width=width, eps=1e-5, bigram=BigramConfig(buckets, 37, 11), loop=LoopConfig(*loop),
                          layers=tuple(RobuvikLayerConfig(att, DenseConfig(ff)) if i % 2 == 0 else RobuvikLayerConfig(lat, moe)
                                       for i in range(layers)))
 

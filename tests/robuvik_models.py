@@ -49,7 +49,7 @@ RC = RobuvikConfig(vocab=101, width=50, eps=1e-5, bigram=BigramConfig(13, 1, 101
     L(LAT(2, 6, 4, 5, 9, 7, 0.4, RotConfig(20.0, 4, None)), DenseConfig(27)),
 ))
 
-RD = RobuvikConfig(vocab=120, width=64, eps=1e-5, bigram=BigramConfig(1021, 31, 7), loop=LoopConfig(1, 2, 2), layers=(
+RD = RobuvikConfig(vocab=120, width=64, eps=1e-5, bigram=BigramConfig(1019, 29, 11), loop=LoopConfig(1, 2, 2), layers=(
     L(ATT(2, 1, 136, 24, 0.1, RotConfig(5000.0, 64, YarnScaling(2.0, 64.0, 16.0, 1.0)), 40), None),
     L(LAT(2, 24, 16, 16, 200, 32, 0.12, RotConfig(200.0, 16, YarnScaling(2.0, 64.0, 16.0, 1.0))), DenseConfig(64)),
     L(ATT(2, 2, 136, 24, 0.1, None, 7), ExpertsConfig(2, 1, 16, None)),
