@@ -50,6 +50,10 @@ struct QkvRopeArgs {
   // the gate of the EPI_SWIGLU epilogue, one of common.h's (0 = silu(g) u), and the clamped gate's limit
   int gate_kind;
   float gate_limit;
+  // EPI_QKV_ROPE: a bias over the (Hq + 2 Hk) D outputs, added to the sums before the rotation (null: none), and
+  // what sine and cosine are multiplied by (1: a plain rotation)
+  const float* bias;
+  float magnitude;
 };
 
 // Routed experts through gemm_wide_kernel: the rows of a workgroup are a tile of one expert's rows, from lists
@@ -82,6 +86,7 @@ struct QkvLane {
   float pos[MT];
   int slot[MT];
   float freq[4];
+  float bias[4];
 };
 
 template <int MT>
@@ -98,6 +103,11 @@ __device__ __forceinline__ QkvLane<MT> load_qkv_lane(const QkvRopeArgs& qa, int 
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) ql.freq[r] = rotated ? qa.inv_freq[t8 * 8 + 4 * (g & 1) + r] : 0.f;
+  // (the lane's four outputs: dims t8 * 8 + 4 (g & 1) .. of the head, or their partners half a head further)
+  const bool in_range = head < qa.Hq + 2 * qa.Hk;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    ql.bias[r] = qa.bias && in_range ? qa.bias[(size_t)head * qa.D + t8 * 8 + 4 * (g & 1) + (g >= 2 ? qa.D >> 1 : 0) + r] : 0.f;
   return ql;
 }
 
@@ -184,12 +194,14 @@ __device__ __forceinline__ void store_tiles(floatx4_t (&acc)[RT][MT], TC* __rest
       float o[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float own = acc[0][mt][r];
+        const float own = acc[0][mt][r] + ql.bias[r];
         const uint32_t u = __float_as_uint(own);
         const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
         const float partner = __uint_as_float(upper ? sw[0] : sw[1]);
         float sn, cs;
         sincos_reduced(ql.pos[mt] * ql.freq[r], &sn, &cs);
+        sn *= qa.magnitude;
+        cs *= qa.magnitude;
         // lower: a cos - b sin with a = own; upper: b cos + a sin with b = own
         o[r] = rotated ? (upper ? own * cs + partner * sn : own * cs - partner * sn) : own;
       }
@@ -1133,10 +1145,13 @@ extern "C" int sa_gemm_bf16_skinny_swiglu(const void* A, const void* W, void* C,
 // Needs D % 16 == 0.
 extern "C" int sa_gemm_bf16_qkv_rope(const void* A, const void* W, void* Q, const int* positions,
                                      const float* inv_freq, const int* slots, void* k_pages, void* v_pages,
-                                     int M, int K, int Hq, int Hk, int D, int page_size, hipStream_t stream) {
+                                     int M, int K, int Hq, int Hk, int D, int page_size, const float* bias,
+                                     float magnitude, hipStream_t stream) {
   if (M <= 0) return 0;
   if (K <= 0 || (K & 7) || Hq <= 0 || Hk <= 0 || D <= 0 || (D & 15) || page_size <= 0) return SA_ERR_ARG;
-  const QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
+  QkvRopeArgs qa = {positions, inv_freq, slots, (bf16_t*)k_pages, (bf16_t*)v_pages, Hq, Hk, D, page_size};
+  qa.bias = bias;
+  qa.magnitude = magnitude;
   if (takes_wide<bf16_t, EPI_QKV_ROPE>(M, 0, K, 1)) return pick_wide<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   if (!takes_skinny<bf16_t, EPI_QKV_ROPE>(M, 0, qa)) return pick_mid<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);
   return pick_skinny<bf16_t, EPI_QKV_ROPE>(A, W, Q, M, (Hq + 2 * Hk) * D, K, 0, 1, qa, stream);

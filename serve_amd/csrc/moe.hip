@@ -396,7 +396,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(const bf16_t* __restrict_
   }
 }
 
-// combine: grid (T).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate);
+// combine: grid (T, parts of a row).  shared: [parts, T, d] (TS), or null; sg: logits fp32, row stride ldz (null: no gate);
 // wts null: the rows are added as they are (their weights went into the experts' inputs).
 // TOPMAX / PMAX: upper bounds of `top` / `parts` (0: any number, in a loop): with bounds, all loads of an output
 // are issued before anything is added (rows beyond the bounds are read from a clamped place and dropped).
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     float wk[TOPMAX > 0 ? TOPMAX : 1];
 #pragma unroll
     for (int k = 0; k < TOPMAX; ++k) wk[k] = k < top ? (wts ? wts[(size_t)t * top + k] : 1.f) : 0.f;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += blockDim.x * gridDim.y) {
       float a[TOPMAX > 0 ? TOPMAX : 1], sp[PMAX];
 #pragma unroll
       for (int k = 0; k < TOPMAX; ++k) a[k] = yk[((size_t)t * top + min(k, top - 1)) * d + i];
@@ -428,7 +428,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     }
     return;
   }
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += blockDim.x * gridDim.y) {
     float v = 0.f;
     for (int k = 0; k < top; ++k) v += (wts ? wts[(size_t)t * top + k] : 1.f) * yk[((size_t)t * top + k) * d + i];
     if (shared) {
@@ -560,7 +560,9 @@ extern "C" int sa_moe_combine(const float* yk, const float* wts, const void* sha
   if (T <= 0) return 0;
   if (top <= 0 || d <= 0 || parts < 1) return SA_ERR_ARG;
   const size_t part_stride = (size_t)T * d;
-  dim3 grid(T), block(d >= 256 ? 256 : 64);
+  // a step of few rows: a value a thread, so that a row's loads are not a chain in one workgroup
+  const int threads = d >= 256 ? 256 : 64;
+  dim3 grid(T, T <= 64 ? (unsigned)((d + threads - 1) / threads) : 1u), block(threads);
 #define GO(TS, TOPMAX, PMAX)                                                                                       \
   hipLaunchKernelGGL((moe_combine_kernel<TS, TOPMAX, PMAX>), grid, block, 0, stream, yk, wts, (const TS*)shared,     \
                      parts, part_stride, sg, ldz, y, top, d)

@@ -1361,10 +1361,14 @@ def qkv_rope_available(a: torch.Tensor, w_qkv: torch.Tensor, k_pages: torch.Tens
 
 def qkv_rope_bf16(a: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
                   inv_freq: torch.Tensor, slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
-                  num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
-    """q, k, v = a @ w_qkv^T (w_qkv = [Wq; Wk; Wv]); q and k rotated by position; q to q_out
-    [M, Hq D], rotated k and v into the cache pages at each token's slot.  One kernel."""
-    _dev(a, w_qkv, q_out, positions, inv_freq, slots, k_pages, v_pages)
+                  num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                  bias: Optional[torch.Tensor] = None, magnitude: float = 1.0) -> torch.Tensor:
+    """q, k, v = a @ w_qkv^T (w_qkv = [Wq; Wk; Wv]) (+ bias, fp32 over the (Hq + 2 Hk) D outputs, added to the fp32
+    sums); q and k rotated by position (sine and cosine times `magnitude`); q to q_out [M, Hq D], rotated k and v
+    into the cache pages at each token's slot.  One kernel."""
+    _dev(a, w_qkv, q_out, positions, inv_freq, slots, k_pages, v_pages, bias)
+    if bias is not None:
+        _f32vec(bias, (num_heads + 2 * num_kv_heads) * head_dim, "bias")
     M, K = a.shape
     Hq, Hk, D = num_heads, num_kv_heads, head_dim
     _check(qkv_rope_available(a, w_qkv, k_pages, D, D, False), "qkv_rope_bf16 does not take these operands")
@@ -1379,7 +1383,8 @@ def qkv_rope_bf16(a: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor, pos
     lib = load_library("gemm_mfma")
     _ret(lib.sa_gemm_bf16_qkv_rope(_ptr(a), _ptr(w_qkv), _ptr(q_out), _ptr(positions), _ptr(inv_freq), _ptr(slots),
                                    _ptr(k_pages), _ptr(v_pages), c_int(M), c_int(K), c_int(Hq), c_int(Hk),
-                                   c_int(D), c_int(page_size), _stream()), "qkv_rope_bf16")
+                                   c_int(D), c_int(page_size), _ptr(bias), c_float(magnitude), _stream()),
+         "qkv_rope_bf16")
     return q_out
 
 

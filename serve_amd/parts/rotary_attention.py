@@ -110,8 +110,17 @@ class RotaryAttention(Part):
         if cache.k_pages.shape[-1] != Dp:
             raise ValueError(f"the cache keeps heads of {cache.k_pages.shape[-1]}, this layer works on {Dp}")
         with trace.span("write_to_cache"):
-            z = linear(h, self.w_in)
             q = self.rt.empty((T, H * Dp))
+            if (writes_cache and D == Dv == Dp and self.rot_dim == D
+                    and ops.qkv_rope_available(h, self.w_in, cache.k_pages, D, self.rot_dim, self.adjacent)):
+                # few rows, whole heads rotated, keys and values of one size: product, biases, rotation and cache
+                # write are one kernel (the biases join the fp32 sums)
+                ops.qkv_rope_bf16(h, self.w_in, q, ctx.positions, self.inv_freq, grp.slots, cache.k_pages,
+                                  cache.v_pages, H, G, D, cache.page_size, self.b_in, self.magnitude)
+                z = None
+            else:
+                z = linear(h, self.w_in)
+        if z is not None:
             ops.bias_rope_kv_write(z, q, ctx.positions, grp.slots if writes_cache else None, cache.k_pages,
                                    cache.v_pages, self.b_in, self.inv_freq, self.rot_dim, self.adjacent, self.magnitude,
                                    H, G, D, Dv)

@@ -12,6 +12,8 @@ The models differ in every size and option:
   RC  width 50 (no multiple of 8), vocabulary 101; both layers run three times; 3 heads on 3, keys 10 / values 7, 4
       rotated dims, a window of 33; latent attention 2 heads of 6 + 4, values 5, latents 9 / 7; experts of width 9
   RE  RB with its first two layers run twice (a loop without a pair table)
+  RF  two attention layers whose heads are rotated whole, keys and values 32 / 32 and 16 / 16, with and without window and
+      stretching: the shapes whose single tokens take the fused product in bfloat16
   RD  sizes above what the matrix-core attention takes: keys 136 / values 24; a latent row of 200 + 16; a single layer
       that runs twice between two that run once
 """
@@ -58,7 +60,14 @@ RD = RobuvikConfig(vocab=120, width=64, eps=1e-5, bigram=BigramConfig(1019, 29, 
 # RB with its first two layers run twice: passes that add the output of an embedding without a pair table
 RE = RobuvikConfig(vocab=RB.vocab, width=RB.width, eps=RB.eps, bigram=None, loop=LoopConfig(0, 2, 2), layers=RB.layers)
 
-MODELS = {"RA": (RA, 3), "RB": (RB, 4), "RC": (RC, 5), "RD": (RD, 6), "RE": (RE, 7)}
+# whole heads rotated, keys and values of one size that is a multiple of 16: in bfloat16, steps of few rows take the
+# product whose epilogue adds the biases, rotates and writes the cache
+RF = RobuvikConfig(vocab=130, width=64, eps=1e-5, bigram=BigramConfig(61, 3, 5), loop=LoopConfig(0, 1, 2), layers=(
+    L(ATT(4, 2, 32, 32, 0.18, RotConfig(300.0, 32, YarnScaling(3.0, 24.0, 6.0, 1.0)), 9), DenseConfig(72)),
+    L(ATT(3, 1, 16, 16, 0.25, RotConfig(40.0, 16, None), None), ExpertsConfig(4, 2, 24, None)),
+))
+
+MODELS = {"RA": (RA, 3), "RB": (RB, 4), "RC": (RC, 5), "RD": (RD, 6), "RE": (RE, 7), "RF": (RF, 8)}
 
 # tables and the output matrix at a scale at which the stream and the logits are of order one
 BASE = {r"^embed$": 40.0, r"^bigram$": 25.0, r"^head$": 6.0, r"^loop\.step$": 2.0}

@@ -18,7 +18,7 @@ from tests.plain import robuvik_plain as rp
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-NAMES = ["RA", "RB", "RC", "RD"]
+NAMES = ["RA", "RB", "RC", "RD", "RF"]
 
 
 def tokens_for(n, seed, vocab):
@@ -409,6 +409,42 @@ def test_bias_rope_kv_write(dtype, H, G, D, Dv, Dp, rot, adjacent, T):
         ops.bias_rope_kv_write(z, q2, pos, None, None, None, bias if with_bias else None, inv if rot else None, rot,
                                adjacent, mag, H, G, D, Dv)
         assert torch.equal(q2, q)
+
+
+@pytest.mark.parametrize("M", [1, 5, 40, 128])
+@pytest.mark.parametrize("H,G,D", [(4, 2, 32), (3, 1, 16), (8, 2, 64), (2, 2, 128)])
+def test_fused_product_with_biases_and_a_stretched_rotation(M, H, G, D):
+    """The bfloat16 product whose epilogue adds biases to the fp32 sums, rotates whole heads with a magnitude and
+    writes queries, keys and values to their places, against the plain computation."""
+    from serve_amd import ops
+    K, page, P = 64, 4, 40
+    g = torch.Generator().manual_seed(M + D)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn((H + 2 * G) * D, K, generator=g) / K ** 0.5).to(torch.bfloat16).cuda()
+    bias = torch.randn((H + 2 * G) * D, generator=g).cuda()
+    pos = torch.tensor([(7 * t) % 150 for t in range(M)], dtype=torch.int32, device="cuda")
+    slot_l = [-1 if t % 11 == 3 else t + 6 for t in range(M)]
+    slots = torch.tensor(slot_l, dtype=torch.int32, device="cuda")
+    f, mag = rp.rotary_frequencies(D, 100.0, {"factor": 3.0, "original": 16.0, "fast": 4.0, "slow": 1.0})
+    assert ops.qkv_rope_available(a, w, torch.empty(0, dtype=torch.bfloat16, device="cuda"), D, D, False)
+    k_pages = torch.full((P, G, page, D), 9.0, dtype=torch.bfloat16, device="cuda")
+    v_pages = torch.full((P, G, D, page), 9.0, dtype=torch.bfloat16, device="cuda")
+    q = torch.empty((M, H * D), dtype=torch.bfloat16, device="cuda")
+    ops.qkv_rope_bf16(a, w, q, pos, f.float().cuda(), slots, k_pages, v_pages, H, G, D, page, bias, mag)
+    z = a.double().cpu() @ w.double().cpu().T + bias.double().cpu()
+    wq = rp.rotate(z[:, : H * D].reshape(M, H, D), pos.cpu(), f, mag, "half")
+    wk = rp.rotate(z[:, H * D: (H + G) * D].reshape(M, G, D), pos.cpu(), f, mag, "half")
+    wv = z[:, (H + G) * D:].reshape(M, G, D)
+    tol = dict(atol=3e-2, rtol=2e-2)
+    assert torch.allclose(q.view(M, H, D).double().cpu(), wq, **tol)
+    stored = [t for t in range(M) if slot_l[t] >= 0]
+    st = torch.tensor([slot_l[t] for t in stored])
+    assert torch.allclose(k_pages.double().cpu()[st // page, :, st % page], wk[stored], **tol)
+    assert torch.allclose(v_pages.double().cpu()[st // page, :, :, st % page], wv[stored], **tol)
+    used = torch.zeros(P * page, dtype=torch.bool)
+    used[st] = True
+    free = (~used).nonzero()[:, 0]
+    assert (k_pages.cpu()[free // page, :, free % page] == 9).all() and (v_pages.cpu()[free // page, :, :, free % page] == 9).all()
 
 
 def _plain_experts(h, router_w, wg, wu, wd, top):
