@@ -18,7 +18,10 @@ Roles and what each must offer:
                 for per-request state of fixed size (`state_request`).
 * feed_forward  `forward(h, ctx) -> delta [T, d]`.
 * embedding     `forward(ctx) -> x` fp32 [T, d] from the step's token ids (and whatever else of
-                the step it needs: positions for a learned position table).
+                the step it needs: positions for a learned position table).  An embedding that looks
+                back at a request's earlier tokens offers `state_request()` and is then called as
+                `forward(ctx, cache, keep=False)`: `cache.state` holds its row per request, and with
+                `keep` it returns (x, a second copy of x) for a run order that adds it again.
 * lm_head       `forward(h) -> logits` fp32 [R, V]; a head with `accepts_out = True` also takes
                 `out=`, a buffer of that shape to write them into (replayed steps bring one).
 * arrangement   puts named parts together into a layer: `PART_ROLES` (name -> role) says which
